@@ -11,10 +11,11 @@ from .spec import LayerSpec, ModelSpec, PartSpec, RunEntry
 from .qwen3 import Qwen3Config
 from .kakunex import KakunexConfig
 from .fimolix import FimolixConfig
+from .reselorn import ReselornConfig
 from .presets import PRESETS, preset
 
 __all__ = [
     "ARCHITECTURES", "architecture_name", "config_from_dict", "load_config", "load_config_dict",
     "register_architecture", "unregister_architecture", "LayerSpec", "ModelSpec", "PartSpec",
-    "RunEntry", "Qwen3Config", "KakunexConfig", "FimolixConfig", "PRESETS", "preset",
+    "RunEntry", "Qwen3Config", "KakunexConfig", "FimolixConfig", "ReselornConfig", "PRESETS", "preset",
 ]

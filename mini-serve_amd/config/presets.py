@@ -116,6 +116,36 @@ def _fimolix_tiny() -> dict:
 PRESETS["fimolix-tiny"] = _fimolix_tiny()
 
 
+def _reselorn_tiny() -> dict:
+    """Four layers that hold every part of the architecture once: a dense layer that makes the first values, a mixture
+    with a shared expert whose values are blended, a layer that neither blends nor has a feed-forward and sees every
+    earlier token, and a mixture without a shared expert behind a rotation that is not slowed down."""
+    slowed = {"base": 3000.0, "dims": 12, "scaling": {"factor": 8.0, "original": 48, "fast": 6.0, "slow": 0.5}}
+
+    def attention(heads, kv_heads, dim, rot, size, v_mix, mlp):
+        m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": 24, "scale": dim ** -0.5, "rot": rot, "v_mix": v_mix}
+        if size:
+            m["mask"] = {"size": size}
+        return {"type": "attention", "mixer": m, "mlp": mlp}
+
+    def moe(experts, top, ff, shared):
+        out = {"kind": "moe", "router": {"experts": experts, "top": top}, "expert": {"ff": ff}}
+        if shared:
+            out["shared"] = {"ff": shared}
+        return out
+
+    return {
+        "architecture": "Reselorn", "vocab": 311, "width": 96, "norm": {"eps": 1e-5},
+        "layers": [attention(4, 2, 32, slowed, 24, True, {"kind": "dense", "ff": 160}),
+                   attention(6, 2, 16, slowed, 40, True, moe(6, 2, 48, 80)),
+                   attention(2, 1, 48, {"base": 100.0, "dims": 48}, 0, False, None),
+                   attention(4, 2, 32, {"base": 3000.0, "dims": 12}, 24, True, moe(5, 3, 32, None))],
+    }
+
+
+PRESETS["reselorn-tiny"] = _reselorn_tiny()
+
+
 def preset(name: str) -> dict:
     try:
         return copy.deepcopy(PRESETS[name])

@@ -323,20 +323,22 @@ extern "C" int ms_cast(const void* in, int in_is_bf16, void* out, int out_is_bf1
 // a row, sin(a) in the second, a = float(pos[t]) * inv_freq[j]. Made once per step and read by every
 // layer's rotation kernel.
 __global__ void rope_table_kernel(const int* __restrict__ pos, const float* __restrict__ inv_freq, float* __restrict__ out,
-                                  int tokens, int half) {
+                                  int tokens, int half, float magnitude) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= tokens * half) return;
   const int t = i / half, j = i % half;
   float sn, cs;
   sincosf((float)pos[t] * inv_freq[j], &sn, &cs);
-  out[(size_t)t * 2 * half + j] = cs;
-  out[(size_t)t * 2 * half + half + j] = sn;
+  out[(size_t)t * 2 * half + j] = cs * magnitude;
+  out[(size_t)t * 2 * half + half + j] = sn * magnitude;
 }
 
-extern "C" int ms_rope_table(const int* pos, const float* inv_freq, float* out, int tokens, int half, hipStream_t st) {
+// `magnitude` multiplies every cosine and sine (1: a plain rotation).
+extern "C" int ms_rope_table(const int* pos, const float* inv_freq, float* out, int tokens, int half, float magnitude,
+                             hipStream_t st) {
   if (tokens <= 0 || half <= 0) return MS_OK;
   if ((long long)tokens * half > 0x7fffffffLL) return MS_BAD_ARG;
-  rope_table_kernel<<<(tokens * half + 255) / 256, 256, 0, st>>>(pos, inv_freq, out, tokens, half);
+  rope_table_kernel<<<(tokens * half + 255) / 256, 256, 0, st>>>(pos, inv_freq, out, tokens, half, magnitude);
   return launch_status();
 }
 

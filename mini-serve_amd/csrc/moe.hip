@@ -1,0 +1,342 @@
+// A mixture of gated feed-forward experts: routing, a plan that sorts the step's (token, chosen expert) pairs by expert,
+// the two products per expert over the sorted pairs, and the weighted sum back into the stream.
+//
+// A step of T tokens that each choose `top` of E experts has P = T top pairs; pair p = t * top + j is token t's j-th
+// choice (largest logit first). The plan cuts every expert's run of pairs into tiles of `tile_rows` pairs; the product
+// kernels are launched over the most tiles a step can have (ceil(P / tile_rows) + min(E, P)) and a block whose tile
+// holds no pair leaves at once: nothing is read back to the host, and a captured step replays.
+//
+// A pair's result depends on its own row and its expert's weights alone (every output element is one dot product, summed
+// in an order that its place in a tile does not change), so neither the order of the pairs inside an expert's run nor
+// what else the step holds changes a token's result; the sum over a token's choices runs in the order of the choices.
+#include "common.h"
+
+#define MOE_MAX_EXPERTS 512
+#define MOE_MAX_TOP WAVE
+
+// ---------------------------------------------------------------------------------------------
+// Routing: z = logits[t] + bias; the `top` largest z (ties: the lower index), largest first; weights = softmax over
+// those alone. One wave per token.
+template <typename TB>
+__global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits, int ld, const TB* __restrict__ bias,
+                                                        int T, int E, int top, int* __restrict__ ids, float* __restrict__ weights) {
+  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+  const int t = blockIdx.x * 4 + wave;
+  if (t >= T) return;
+  float z[MOE_MAX_EXPERTS / WAVE];
+#pragma unroll
+  for (int i = 0; i < MOE_MAX_EXPERTS / WAVE; ++i) {
+    const int e = lane + i * WAVE;
+    z[i] = e < E ? logits[(size_t)t * ld + e] + (bias ? to_f32(bias[e]) : 0.f) : -INFINITY;
+  }
+  float chosen = 0.f;  // lane j keeps the j-th chosen logit
+  for (int j = 0; j < top; ++j) {
+    float best = -INFINITY;
+    int at = 0x7fffffff;
+#pragma unroll
+    for (int i = 0; i < MOE_MAX_EXPERTS / WAVE; ++i)
+      if (z[i] > best) { best = z[i]; at = lane + i * WAVE; }  // taken and absent experts hold -inf
+#pragma unroll
+    for (int off = WAVE / 2; off > 0; off >>= 1) {
+      const float ob = __shfl_xor(best, off, WAVE);
+      const int oa = __shfl_xor(at, off, WAVE);
+      if (ob > best || (ob == best && oa < at)) { best = ob; at = oa; }
+    }
+    if (at >= E) at = j;  // logits that are no numbers: nothing to choose by, but the plan needs an expert that exists
+#pragma unroll
+    for (int i = 0; i < MOE_MAX_EXPERTS / WAVE; ++i)
+      if (lane + i * WAVE == at) z[i] = -INFINITY;
+    if (lane == 0) ids[(size_t)t * top + j] = at;
+    if (lane == j) chosen = best;
+  }
+  // every chosen logit is at most the first; the sum runs in the order of the choices
+  const float m = __shfl(chosen, 0, WAVE);
+  float sum = 0.f;
+  for (int j = 0; j < top; ++j) sum += expf(__shfl(chosen, j, WAVE) - m);
+  if (lane < top) weights[(size_t)t * top + lane] = expf(chosen - m) / sum;
+}
+
+extern "C" int ms_moe_route(const float* logits, int ld, const void* bias, int bias_is_bf16, int T, int E, int top, int* ids,
+                            float* weights, hipStream_t st) {
+  if (T <= 0) return MS_OK;
+  if (logits == nullptr || ids == nullptr || weights == nullptr || E < 1 || top < 1 || top > E || ld < E) return MS_BAD_ARG;
+  if (E > MOE_MAX_EXPERTS || top > MOE_MAX_TOP) return MS_UNSUPPORTED;
+  const unsigned blocks = (unsigned)((T + 3) / 4);
+  if (bias_is_bf16) moe_route_kernel<bf16><<<blocks, 256, 0, st>>>(logits, ld, (const bf16*)bias, T, E, top, ids, weights);
+  else moe_route_kernel<float><<<blocks, 256, 0, st>>>(logits, ld, (const float*)bias, T, E, top, ids, weights);
+  return launch_status();
+}
+
+// ---------------------------------------------------------------------------------------------
+// The plan, one block: counts per expert, every expert's run of `order` (order[i] = the pair at sorted place i), and the
+// tiles: tile n covers places tile_start[n] .. tile_start[n] + tile_count[n] - 1 of expert tile_expert[n]. Tiles past the
+// last get a count of zero.
+__global__ __launch_bounds__(1024) void moe_plan_kernel(const int* __restrict__ ids, int P, int E, int tile_rows, int max_tiles,
+                                                        int* __restrict__ order, int* __restrict__ tile_expert,
+                                                        int* __restrict__ tile_start, int* __restrict__ tile_count) {
+  __shared__ int counts[MOE_MAX_EXPERTS], offsets[MOE_MAX_EXPERTS], cursor[MOE_MAX_EXPERTS], tile_base[MOE_MAX_EXPERTS];
+  __shared__ int total_tiles;
+  const int tid = threadIdx.x;
+  for (int e = tid; e < E; e += 1024) { counts[e] = 0; cursor[e] = 0; }
+  __syncthreads();
+  for (int p = tid; p < P; p += 1024) atomicAdd(&counts[min(max(ids[p], 0), E - 1)], 1);
+  __syncthreads();
+  if (tid == 0) {
+    int off = 0, nt = 0;
+    for (int e = 0; e < E; ++e) {
+      offsets[e] = off;
+      tile_base[e] = nt;
+      off += counts[e];
+      nt += (counts[e] + tile_rows - 1) / tile_rows;
+    }
+    total_tiles = nt;
+  }
+  __syncthreads();
+  for (int e = tid; e < E; e += 1024) {
+    const int n = (counts[e] + tile_rows - 1) / tile_rows;
+    for (int i = 0; i < n; ++i) {
+      const int at = tile_base[e] + i;
+      if (at >= max_tiles) break;
+      tile_expert[at] = e;
+      tile_start[at] = offsets[e] + i * tile_rows;
+      tile_count[at] = min(tile_rows, counts[e] - i * tile_rows);
+    }
+  }
+  for (int n = total_tiles + tid; n < max_tiles; n += 1024) {
+    tile_expert[n] = 0;
+    tile_start[n] = 0;
+    tile_count[n] = 0;
+  }
+  for (int p = tid; p < P; p += 1024) {
+    const int e = min(max(ids[p], 0), E - 1);
+    order[offsets[e] + atomicAdd(&cursor[e], 1)] = p;
+  }
+}
+
+extern "C" int ms_moe_plan(const int* ids, int P, int E, int tile_rows, int max_tiles, int* order, int* tile_expert,
+                           int* tile_start, int* tile_count, hipStream_t st) {
+  if (P <= 0) return MS_OK;
+  if (ids == nullptr || order == nullptr || tile_expert == nullptr || tile_start == nullptr || tile_count == nullptr || E < 1 ||
+      tile_rows < 1 || max_tiles < (P + tile_rows - 1) / tile_rows + (E < P ? E : P))
+    return MS_BAD_ARG;
+  if (E > MOE_MAX_EXPERTS) return MS_UNSUPPORTED;
+  moe_plan_kernel<<<1, 1024, 0, st>>>(ids, P, E, tile_rows, max_tiles, order, tile_expert, tile_start, tile_count);
+  return launch_status();
+}
+
+// ---------------------------------------------------------------------------------------------
+// The experts' products on the matrix cores (bfloat16 operands, float32 sums, v_mfma_f32_16x16x32_bf16), operands
+// straight from memory, 16 bytes a lane. A wave owns 16 pairs x 64 columns; a block's four waves split a tile of 64 pairs
+// by rows (64 columns a block), a tile of 16 pairs by columns (256 columns a block: steps of few tokens, where every
+// chosen expert has a tile of its own and its weights are streamed once).
+//   GATED: rows are x[token of the pair] (K = the model's width), two weights per expert, gate and up [E, N, K]; the result
+//          act(gate) * up goes to h[sorted place][N] in the compute type.
+//   else:  rows are h[sorted place] (K = the experts' width), one weight per expert [E, N, K]; the result times the pair's
+//          routing weight goes to y[pair][N] in float32.
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 moe_bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float moe_floatx4;
+
+// Eight consecutive elements from p + k, those at or past K zero. ALIGNED: one 16-byte load (K, the row strides and the
+// bases are multiples of 8 elements, so a lane's eight are all inside or all outside).
+template <bool ALIGNED> __device__ __forceinline__ moe_bf16x8 moe_load(const bf16* p, int k, int K, bool ok) {
+  union { uint4 u; moe_bf16x8 v; bf16 e[8]; } x;
+  x.u = make_uint4(0, 0, 0, 0);
+  if (ALIGNED) {
+    if (ok && k < K) x.u = *reinterpret_cast<const uint4*>(p + k);
+  } else if (ok) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+      if (k + i < K) x.e[i] = p[k + i];
+  }
+  return x.v;
+}
+
+template <bool GATED, bool ALIGNED>
+__global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(
+    const bf16* __restrict__ a, int lda, const bf16* __restrict__ w1, const bf16* __restrict__ w2, void* __restrict__ out,
+    const int* __restrict__ order, const int* __restrict__ tile_expert, const int* __restrict__ tile_start,
+    const int* __restrict__ tile_count, const float* __restrict__ pair_weight, int top, int N, int K, int tile_rows, int act) {
+  const int count = tile_count[blockIdx.x];
+  if (count == 0) return;
+  const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE, l16 = lane % 16, grp = lane / 16;
+  const bool by_rows = tile_rows == 64;
+  const int m0 = by_rows ? wave * 16 : 0;
+  const int n0 = by_rows ? blockIdx.y * 64 : blockIdx.y * 256 + wave * 64;
+  if (m0 >= count || n0 >= N) return;
+  const int e = tile_expert[blockIdx.x], start = tile_start[blockIdx.x];
+  const bool row_ok = m0 + l16 < count;
+  const int place = start + m0 + (row_ok ? l16 : 0);
+  const bf16* ap = a + (size_t)(GATED ? order[place] / top : place) * lda;
+  const bf16* wp1[4];
+  const bf16* wp2[4];
+  bool col_ok[4];
+#pragma unroll
+  for (int nt = 0; nt < 4; ++nt) {
+    col_ok[nt] = n0 + nt * 16 + l16 < N;
+    const size_t at = ((size_t)e * N + (col_ok[nt] ? n0 + nt * 16 + l16 : 0)) * K;
+    wp1[nt] = w1 + at;
+    wp2[nt] = GATED ? w2 + at : nullptr;
+  }
+  moe_floatx4 acc1[4], acc2[4];
+#pragma unroll
+  for (int nt = 0; nt < 4; ++nt) acc1[nt] = acc2[nt] = moe_floatx4{0.f, 0.f, 0.f, 0.f};
+  for (int k0 = 0; k0 < K; k0 += 32) {
+    const int kk = k0 + grp * 8;  // the lane's eight elements of this step
+    const moe_bf16x8 av = moe_load<ALIGNED>(ap, kk, K, row_ok);
+    moe_bf16x8 b1[4], b2[4];
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt) {
+      b1[nt] = moe_load<ALIGNED>(wp1[nt], kk, K, col_ok[nt]);
+      if (GATED) b2[nt] = moe_load<ALIGNED>(wp2[nt], kk, K, col_ok[nt]);
+    }
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt) {
+      acc1[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, b1[nt], acc1[nt], 0, 0, 0);
+      if (GATED) acc2[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, b2[nt], acc2[nt], 0, 0, 0);
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int m = m0 + grp * 4 + r;
+    if (m >= count) continue;
+    if (GATED) {
+      bf16* o = (bf16*)out + (size_t)(start + m) * N + n0 + l16;
+#pragma unroll
+      for (int nt = 0; nt < 4; ++nt)
+        if (col_ok[nt]) o[nt * 16] = static_cast<bf16>(gated_value(acc1[nt][r], acc2[nt][r], act, 0.f));
+    } else {
+      const int pair = order[start + m];
+      const float pw = pair_weight[pair];
+      float* o = (float*)out + (size_t)pair * N + n0 + l16;
+#pragma unroll
+      for (int nt = 0; nt < 4; ++nt)
+        if (col_ok[nt]) o[nt * 16] = acc1[nt][r] * pw;
+    }
+  }
+}
+
+// The same two products in true float32 on the vector units: 64 x 64 tiles through LDS, every output element one chain of
+// fused multiply-adds over k in ascending order.
+template <bool GATED>
+__global__ __launch_bounds__(256) void moe_gemm_f32_kernel(
+    const float* __restrict__ a, int lda, const float* __restrict__ w1, const float* __restrict__ w2, float* __restrict__ out,
+    const int* __restrict__ order, const int* __restrict__ tile_expert, const int* __restrict__ tile_start,
+    const int* __restrict__ tile_count, const float* __restrict__ pair_weight, int top, int N, int K, int act) {
+  const int count = tile_count[blockIdx.x];
+  if (count == 0) return;
+  __shared__ float As[16][64 + 4];
+  __shared__ float W1s[16][64 + 4];
+  __shared__ float W2s[GATED ? 16 : 1][64 + 4];
+  const int tid = threadIdx.x;
+  const int e = tile_expert[blockIdx.x], start = tile_start[blockIdx.x];
+  const int n0 = blockIdx.y * 64;
+  const int tx = tid % 16, ty = tid / 16;      // 16 x 16 threads, 4 x 4 outputs each
+  const int lr = tid / 4, lk = (tid % 4) * 4;  // loader: row within the tile, k offset
+  const bool a_ok = lr < count;
+  const float* arow = a + (size_t)(a_ok ? (GATED ? order[start + lr] / top : start + lr) : 0) * lda;
+  const bool w_ok = n0 + lr < N;
+  const size_t wat = ((size_t)e * N + (w_ok ? n0 + lr : 0)) * K;
+  float acc1[4][4], acc2[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc1[i][j] = acc2[i][j] = 0.f;
+  for (int k0 = 0; k0 < K; k0 += 16) {
+    float av[4], wv1[4], wv2[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int k = k0 + lk + i;
+      av[i] = (a_ok && k < K) ? arow[k] : 0.f;
+      wv1[i] = (w_ok && k < K) ? w1[wat + k] : 0.f;
+      wv2[i] = (GATED && w_ok && k < K) ? w2[wat + k] : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      As[lk + i][lr] = av[i];
+      W1s[lk + i][lr] = wv1[i];
+      if (GATED) W2s[lk + i][lr] = wv2[i];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < 16; ++k) {
+      float x[4], u[4], v[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) x[i] = As[k][ty * 4 + i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        u[j] = W1s[k][tx * 4 + j];
+        v[j] = GATED ? W2s[k][tx * 4 + j] : 0.f;
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          acc1[i][j] = fmaf(x[i], u[j], acc1[i][j]);
+          if (GATED) acc2[i][j] = fmaf(x[i], v[j], acc2[i][j]);
+        }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int m = ty * 4 + i;
+    if (m >= count) continue;
+    const int pair = GATED ? 0 : order[start + m];
+    const float pw = GATED ? 1.f : pair_weight[pair];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = n0 + tx * 4 + j;
+      if (n >= N) continue;
+      if (GATED) out[(size_t)(start + m) * N + n] = gated_value(acc1[i][j], acc2[i][j], act, 0.f);
+      else out[(size_t)pair * N + n] = acc1[i][j] * pw;
+    }
+  }
+}
+
+// a: the rows ([tokens, lda] for the gated product, [P, lda] sorted places for the other); w1 (and w2, gated): [E, N, K];
+// out: h [P, N] (gated, the compute type) or y [P, N] float32. tile_rows: 16 or 64 in bfloat16, 64 in float32.
+extern "C" int ms_moe_gemm(const void* a, int lda, const void* w1, const void* w2, void* out, int is_bf16, int gated,
+                           const int* order, const int* tile_expert, const int* tile_start, const int* tile_count,
+                           const float* pair_weight, int max_tiles, int top, int N, int K, int tile_rows, int act, hipStream_t st) {
+  if (max_tiles <= 0 || N <= 0) return MS_OK;
+  if (a == nullptr || w1 == nullptr || (gated && w2 == nullptr) || out == nullptr || order == nullptr || tile_expert == nullptr ||
+      tile_start == nullptr || tile_count == nullptr || (!gated && pair_weight == nullptr) || top < 1 || K <= 0 || lda < K ||
+      act < 0 || act >= MS_ACT_COUNT)
+    return MS_BAD_ARG;
+  if (is_bf16) {
+    if (tile_rows != 16 && tile_rows != 64) return MS_BAD_ARG;
+    const int cols = tile_rows == 64 ? 64 : 256;
+    const dim3 grid(max_tiles, (N + cols - 1) / cols);
+    if (grid.y > 65535) return MS_BAD_ARG;
+    const bool aligned = K % 8 == 0 && lda % 8 == 0 && (size_t)a % 16 == 0 && (size_t)w1 % 16 == 0 && (!gated || (size_t)w2 % 16 == 0);
+#define MOE(G, A) moe_gemm_bf16_kernel<G, A><<<grid, 256, 0, st>>>((const bf16*)a, lda, (const bf16*)w1, (const bf16*)w2, out, order, tile_expert, tile_start, tile_count, pair_weight, top, N, K, tile_rows, act)
+    if (gated) { if (aligned) MOE(true, true); else MOE(true, false); }
+    else { if (aligned) MOE(false, true); else MOE(false, false); }
+#undef MOE
+  } else {
+    if (tile_rows != 64) return MS_BAD_ARG;
+    const dim3 grid(max_tiles, (N + 63) / 64);
+    if (grid.y > 65535) return MS_BAD_ARG;
+    if (gated) moe_gemm_f32_kernel<true><<<grid, 256, 0, st>>>((const float*)a, lda, (const float*)w1, (const float*)w2, (float*)out, order, tile_expert, tile_start, tile_count, pair_weight, top, N, K, act);
+    else moe_gemm_f32_kernel<false><<<grid, 256, 0, st>>>((const float*)a, lda, (const float*)w1, nullptr, (float*)out, order, tile_expert, tile_start, tile_count, pair_weight, top, N, K, act);
+  }
+  return launch_status();
+}
+
+// ---------------------------------------------------------------------------------------------
+// stream[t][n] += sum over j < top of y[t * top + j][n], in ascending j.
+__global__ void moe_combine_kernel(float* __restrict__ stream, const float* __restrict__ y, int top, int N) {
+  const int n = blockIdx.x * blockDim.x + threadIdx.x;
+  if (n >= N) return;
+  const size_t t = blockIdx.y;
+  float acc = 0.f;
+  for (int j = 0; j < top; ++j) acc += y[(t * top + j) * N + n];
+  stream[t * N + n] += acc;
+}
+
+extern "C" int ms_moe_combine(float* stream, const float* y, int T, int top, int N, hipStream_t st) {
+  if (T <= 0 || N <= 0) return MS_OK;
+  if (stream == nullptr || y == nullptr || top < 1 || T > 65535) return MS_BAD_ARG;
+  moe_combine_kernel<<<dim3((N + 255) / 256, T), 256, 0, st>>>(stream, y, top, N);
+  return launch_status();
+}

@@ -43,7 +43,7 @@ _SIGNATURES = {
     "ms_gated_recurrence_chunk_max_dim": [],
     "ms_gemm_bf16_gated": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
     "ms_cast": [_c_void, _c_int, _c_void, _c_int, _c_ll, _c_void],
-    "ms_rope_table": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_void],
+    "ms_rope_table": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_float, _c_void],
     "ms_qk_norm_rope_store": [_c_void, _c_void, _c_int, _c_ll, _c_void, _c_int, _c_int, _c_void, _c_void, _c_void,
                               _c_int, _c_float, _c_void, _c_int, _c_int, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int,
                               _c_void],
@@ -95,6 +95,14 @@ _SIGNATURES = {
     "ms_sample_scratch_bytes": [_c_int],
     "ms_sample_rows_static": [_c_void, _c_int, _c_int, _c_ll, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void],
     "ms_sample_rows_static_max_rows": [],
+    "ms_head_prepare_store": [_c_void, _c_int, _c_void, _c_int, _c_void, _c_void, _c_void, _c_int, _c_int, _c_float, _c_void, _c_int,
+                              _c_int, _c_void, _c_int, _c_float, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
+                              _c_void],
+    "ms_moe_route": [_c_void, _c_int, _c_void, _c_int, _c_int, _c_int, _c_int, _c_void, _c_void, _c_void],
+    "ms_moe_plan": [_c_void, _c_int, _c_int, _c_int, _c_int, _c_void, _c_void, _c_void, _c_void, _c_void],
+    "ms_moe_gemm": [_c_void, _c_int, _c_void, _c_void, _c_void, _c_int, _c_int, _c_void, _c_void, _c_void, _c_void, _c_void,
+                    _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
+    "ms_moe_combine": [_c_void, _c_void, _c_int, _c_int, _c_int, _c_void],
     "ms_measure_read": [_c_void, _c_ll, _c_int, _c_void, _c_void],
     "ms_measure_copy": [_c_void, _c_void, _c_ll, _c_int, _c_void],
 }
@@ -453,18 +461,96 @@ def add_pending(residual: torch.Tensor, pending: SplitSum | None) -> None:
            "splitk_reduce")
 
 
+# ------------------------------------------------------------------------------------- mixture of experts
+
+MOE_MAX_EXPERTS = 512  # MOE_MAX_EXPERTS in csrc/moe.hip
+MOE_MAX_TOP = 64
+MOE_SMALL_TILE_PAIRS = 16  # (token, expert) pairs per expert, on average, up to which a step runs 16-pair tiles
+
+
+def moe_route(logits: torch.Tensor, bias: torch.Tensor | None, top: int):
+    """Per row of the float32 router logits ``[T, E]`` (plus ``bias [E]``): the ``top`` experts with the largest values,
+    largest first (ties: the lower index), as int32 ``[T, top]``, and the softmax over those values alone, float32
+    ``[T, top]``."""
+    _dev(logits, "logits", F32, 2)
+    t, e = logits.shape
+    if not 1 <= top <= e:
+        raise ValueError(f"top {top} of {e} experts")
+    if e > MOE_MAX_EXPERTS or top > MOE_MAX_TOP:
+        raise ValueError(f"{e} experts / top {top}: the routing kernel takes up to {MOE_MAX_EXPERTS} experts and {MOE_MAX_TOP} choices")
+    if bias is not None:
+        _dev(bias, "bias", (F32, BF16), 1)
+        if bias.shape[0] != e:
+            raise ValueError(f"the router's bias has {bias.shape[0]} elements for {e} experts")
+    ids = torch.empty((t, top), dtype=I32, device=logits.device)
+    weights = torch.empty((t, top), dtype=F32, device=logits.device)
+    _check(library().ms_moe_route(logits.data_ptr(), e, _ptr(bias), int(bias is not None and bias.dtype == BF16), t, e, top,
+                                  ids.data_ptr(), weights.data_ptr(), _stream()), "moe_route")
+    return ids, weights
+
+
+def moe_experts(x: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, gate: torch.Tensor, up: torch.Tensor,
+                down: torch.Tensor, activation: str, stream: torch.Tensor) -> None:
+    """``stream[t] += sum_j weights[t, j] * down[e] (act(gate[e] x[t]) * (up[e] x[t]))`` with ``e = ids[t, j]``, the sum in
+    ascending ``j``. ``x [T, W]`` in the compute dtype, ``gate`` / ``up`` ``[E, F, W]`` and ``down [E, W, F]`` in the same,
+    ``stream`` float32 ``[T, W]``. The step's (token, expert) pairs are sorted by expert on the device and every expert's
+    run is multiplied in tiles (bfloat16: on the matrix cores; float32: fused multiply-adds in ascending k); the launches
+    cover the most tiles the step can have, so nothing is read back and a captured step replays."""
+    act = _activation(activation)
+    if act >= 2:
+        raise NotImplementedError(f"activation {activation!r} is not of the form act(gate) * up")
+    _dev(x, "x", (F32, BF16), 2)
+    for w, nm in ((gate, "gate"), (up, "up"), (down, "down")):
+        _dev(w, nm, x.dtype, 3)
+    _dev(ids, "ids", I32, 2)
+    _dev(weights, "weights", F32, 2)
+    _dev(stream, "stream", F32, 2)
+    t, width = x.shape
+    e, f = gate.shape[0], gate.shape[1]
+    top = ids.shape[1]
+    if gate.shape != (e, f, width) or up.shape != (e, f, width) or down.shape != (e, width, f):
+        raise ValueError(f"expert weights {tuple(gate.shape)} / {tuple(up.shape)} / {tuple(down.shape)} do not fit x {tuple(x.shape)}")
+    if ids.shape[0] != t or tuple(weights.shape) != tuple(ids.shape) or tuple(stream.shape) != (t, width):
+        raise ValueError("ids, weights and stream must have one row per row of x")
+    if e > MOE_MAX_EXPERTS:
+        raise ValueError(f"{e} experts: the kernels take up to {MOE_MAX_EXPERTS}")
+    if t == 0:
+        return
+    if t > MAX_STEP_TOKENS:
+        raise ValueError(f"{t} rows: one launch takes at most {MAX_STEP_TOKENS}")
+    pairs = t * top
+    bf = x.dtype == BF16
+    tile_rows = 16 if bf and pairs <= MOE_SMALL_TILE_PAIRS * e else 64
+    max_tiles = -(-pairs // tile_rows) + min(e, pairs)
+    dev = x.device
+    order = torch.empty((pairs,), dtype=I32, device=dev)
+    tiles = torch.empty((3, max_tiles), dtype=I32, device=dev)
+    lib = library()
+    _check(lib.ms_moe_plan(ids.data_ptr(), pairs, e, tile_rows, max_tiles, order.data_ptr(), tiles[0].data_ptr(), tiles[1].data_ptr(),
+                           tiles[2].data_ptr(), _stream()), "moe_plan")
+    plan = (order.data_ptr(), tiles[0].data_ptr(), tiles[1].data_ptr(), tiles[2].data_ptr())
+    h = torch.empty((pairs, f), dtype=x.dtype, device=dev)
+    _check(lib.ms_moe_gemm(x.data_ptr(), width, gate.data_ptr(), up.data_ptr(), h.data_ptr(), int(bf), 1, *plan, None, max_tiles, top,
+                           f, width, tile_rows, act, _stream()), "moe_gemm")
+    y = torch.empty((pairs, width), dtype=F32, device=dev)
+    _check(lib.ms_moe_gemm(h.data_ptr(), f, down.data_ptr(), None, y.data_ptr(), int(bf), 0, *plan, weights.data_ptr(), max_tiles, top,
+                           width, f, tile_rows, act, _stream()), "moe_gemm")
+    _check(lib.ms_moe_combine(stream.data_ptr(), y.data_ptr(), t, top, width, _stream()), "moe_combine")
+
+
 # ------------------------------------------------------------------------------------- attention
 
 
-def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor) -> torch.Tensor:
-    """Cosines and sines of the rotation angles ``float32(position) * inv_freq[j]`` of a step's tokens:
-    float32 ``[T, 2 * len(inv_freq)]``, a row holding the cosines, then the sines. Made once per step
+def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor, magnitude: float = 1.0) -> torch.Tensor:
+    """Cosines and sines of the rotation angles ``float32(position) * inv_freq[j]`` of a step's tokens, each multiplied
+    by ``magnitude``: float32 ``[T, 2 * len(inv_freq)]``, a row holding the cosines, then the sines. Made once per step
     and shared by all layers that rotate by the same frequencies."""
     _dev(positions, "positions", I32, 1)
     _dev(inv_freq, "inv_freq", F32, 1)
     t, half = positions.shape[0], inv_freq.shape[0]
     out = torch.empty((t, 2 * half), dtype=F32, device=positions.device)
-    _check(library().ms_rope_table(positions.data_ptr(), inv_freq.data_ptr(), out.data_ptr(), t, half, _stream()), "rope_table")
+    _check(library().ms_rope_table(positions.data_ptr(), inv_freq.data_ptr(), out.data_ptr(), t, half, float(magnitude), _stream()),
+           "rope_table")
     return out
 
 
@@ -1119,6 +1205,70 @@ def qkv_norm_rope_store(qkv, slots, q_weight, k_weight, eps, rope, k_cache, v_ca
         float(eps), _ptr(rope), int(rot_dim), pair, _ptr(k_cache) if slots is not None else None,
         _ptr(v_cache) if slots is not None else None, t, num_heads, num_kv_heads, head_dim, int(value_dim), page_size, _stream()),
         "qkv_norm_rope_store")
+    return q_out
+
+
+HEAD_NORMS = {None: 0, "before": 1, "after": 2}  # where a per-head RMS norm sits relative to the rotation (MS_NORM_* in csrc/attention_prep.hip)
+PREPARE_MAX_HEAD_DIM = 1024
+
+
+def head_prepare_store(qkv, slots, norm: str | None, q_weight, k_weight, eps, rope, pairing, k_cache, v_cache, num_heads,
+                       num_kv_heads, head_dim, value_dim, out_dtype, v_first=None, blend: float = 0.0) -> torch.Tensor:
+    """From float32 ``qkv [T, Hq D + Hkv D + Hkv Dv]``: rotation of the first ``rope.shape[1]`` elements of each query and
+    key head, in pairs as ``pairing`` names them, by the angles of ``rope`` (a ``rope_table`` of these tokens; None: no
+    rotation), and an RMS norm per head, ``norm="before"`` the rotation or ``"after"`` it (weights ``[D]`` each, or None for
+    a bare division by the root mean square; ``norm=None``: no norm). ``v_first`` (a float32 tensor of at least ``Hkv Dv``
+    columns, one row per token, possibly a view of wider rows): the values become ``(1 - blend) v + blend v_first``. Keys
+    and values are stored into the cache pages at ``slots`` (skipped when ``slots`` is None). Returns the finished queries
+    ``[T, Hq D]`` in ``out_dtype``."""
+    _dev(qkv, "qkv", F32, 2)
+    t = qkv.shape[0]
+    width = num_heads * head_dim + num_kv_heads * (head_dim + value_dim)
+    if qkv.shape[1] != width:
+        raise ValueError(f"qkv has width {qkv.shape[1]}, expected {width}")
+    if out_dtype not in (F32, BF16):
+        raise TypeError(f"unsupported output dtype {out_dtype}")
+    if norm not in HEAD_NORMS:
+        raise ValueError(f"norm {norm!r}: one of {list(HEAD_NORMS)}")
+    if max(head_dim, value_dim) > PREPARE_MAX_HEAD_DIM or min(head_dim, value_dim) < 1:
+        raise ValueError(f"head sizes {head_dim} / {value_dim} are outside the kernel's range 1..{PREPARE_MAX_HEAD_DIM}")
+    w_bf16 = 0
+    if (q_weight is None) != (k_weight is None) or (q_weight is not None and norm is None):
+        raise ValueError("the query and the key norm's weights come together, and only with a norm")
+    if q_weight is not None:
+        for w, nm in ((q_weight, "q_norm"), (k_weight, "k_norm")):
+            _dev(w, nm, (F32, BF16), 1)
+            if w.shape[0] != head_dim:
+                raise ValueError(f"{nm} weight has {w.shape[0]} elements for head_dim {head_dim}")
+        if q_weight.dtype != k_weight.dtype:
+            raise TypeError("q_norm and k_norm weights differ in dtype")
+        w_bf16 = int(q_weight.dtype == BF16)
+    page_size = 1
+    if slots is not None:
+        _dev(slots, "slots", I32, 1)
+        if slots.shape[0] != t:
+            raise ValueError("one slot per token is needed")
+        page_size = _check_caches(k_cache, v_cache, out_dtype, num_kv_heads, head_dim, value_dim)
+    rot_dim, pair = 0, _pairing(pairing)
+    if rope is not None:
+        _dev(rope, "rope", F32, 2)
+        rot_dim = rope.shape[1]
+        if rope.shape[0] != t or rot_dim % 2 or rot_dim > head_dim or rot_dim < 2:
+            raise ValueError(f"rotation table is {tuple(rope.shape)}; {t} tokens and an even width up to {head_dim} are needed")
+    first_ld = 0
+    if v_first is not None:
+        if not (isinstance(v_first, torch.Tensor) and v_first.is_cuda and v_first.dtype == F32 and v_first.dim() == 2
+                and v_first.stride(1) == 1):
+            raise TypeError("v_first must be float32 rows on the GPU with contiguous elements")
+        if v_first.shape[0] != t or v_first.shape[1] < num_kv_heads * value_dim:
+            raise ValueError(f"v_first is {tuple(v_first.shape)}; {t} rows of at least {num_kv_heads * value_dim} values are needed")
+        first_ld = v_first.stride(0)
+    q_out = torch.empty((t, num_heads * head_dim), dtype=out_dtype, device=qkv.device)
+    _check(library().ms_head_prepare_store(
+        qkv.data_ptr(), qkv.shape[1], q_out.data_ptr(), int(out_dtype == BF16), _ptr(slots), _ptr(q_weight), _ptr(k_weight), w_bf16,
+        HEAD_NORMS[norm], float(eps), _ptr(rope), int(rot_dim), pair, _ptr(v_first), int(first_ld), float(blend),
+        _ptr(k_cache) if slots is not None else None, _ptr(v_cache) if slots is not None else None, t, num_heads, num_kv_heads,
+        head_dim, int(value_dim), page_size, _stream()), "head_prepare_store")
     return q_out
 
 

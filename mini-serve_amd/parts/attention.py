@@ -19,7 +19,16 @@ positions; the cache keeps their pages); ``value_dim`` (size of a value head, de
 ``qk_norm="projection"`` (the RMS norm runs over a token's whole query projection and over its whole key
 projection, before they are split into heads, with weights of those sizes; default ``"head"``);
 ``exact_weights`` (the softmax weights meet the values in float32: no rounding of them to bfloat16 for the
-matrix cores); ``names`` (the tensors' names behind the prefix, by ``q k v o q_norm k_norm``).
+matrix cores); ``names`` (the tensors' names behind the prefix, by ``q k v o q_norm k_norm sink blend``).
+
+And four more, which run the path whose every step between projection and attention is a parameter of one kernel
+(``ops.head_prepare_store``): ``qk_norm="head_rotated"`` (the norm per head sits behind the rotation instead of before
+it: with cosines and sines that carry a magnitude the two differ); ``qk_norm_weights=False`` (the norms have no weights:
+a bare division by the root mean square); ``sinks`` (a learned number per query head, tensor ``[heads]``, whose exponential
+joins the head's softmax denominator with neither key nor value); ``value_blend`` (``"first"``: the layer's values, as
+projected, are kept for the step's later layers; ``"blend"``: its values become ``(1 - a) v + a v_first`` with the one
+learned number ``a`` (tensor ``[]``) and ``v_first`` the values of the same token that the ``"first"`` layer of the same
+``blend_group`` kept; the blend is what is cached and attended over. The two layers' value shapes must agree).
 """
 
 from __future__ import annotations
@@ -37,7 +46,7 @@ def _names(spec: PartSpec) -> dict[str, str]:
     p = spec.get("prefix", "")
     given = spec.get("names") or {}
     default = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight",
-               "q_norm": "q_norm.weight", "k_norm": "k_norm.weight"}
+               "q_norm": "q_norm.weight", "k_norm": "k_norm.weight", "sink": "sinks", "blend": "value_blend"}
     return {k: p + given.get(k, d) for k, d in default.items()}
 
 
@@ -58,22 +67,34 @@ class GQAttention(Mixer):
         self.qk_norm = spec.get("qk_norm", "head")
         self.exact_weights = bool(spec.get("exact_weights", False))
         self.names = _names(spec)
-        if self.qk_norm not in ("head", "projection"):
-            raise ValueError(f"qk_norm {self.qk_norm!r}: 'head' or 'projection'")
+        self.qk_norm_weights = bool(spec.get("qk_norm_weights", True))
+        self.sinks = bool(spec.get("sinks", False))
+        self.value_blend = spec.get("value_blend")
+        self.blend_key = ("value_blend", spec.get("blend_group", "values"))
+        if self.qk_norm not in ("head", "projection", "head_rotated"):
+            raise ValueError(f"qk_norm {self.qk_norm!r}: 'head', 'projection' or 'head_rotated'")
+        if self.value_blend not in (None, "first", "blend"):
+            raise ValueError(f"value_blend {self.value_blend!r}: None, 'first' or 'blend'")
+        # The path on which rotation, norm, blend and store are one kernel with every option a parameter.
+        self.prepared = (self.qk_norm == "head_rotated" or self.sinks or self.value_blend is not None
+                         or (self.qk_norm_eps is not None and not self.qk_norm_weights))
+        if self.prepared and (self.qk_norm == "projection" or self.keep_first):
+            raise NotImplementedError("sinks, blended values and a norm behind the rotation go with a norm per head and no kept first keys")
         if self.keep_first < 0 or self.window < 0:
             raise ValueError("window and keep_first must not be negative")
         # The path with one norm over the projection, values of their own size, kept first keys or unrounded weights.
-        self.wide = (self.qk_norm == "projection" and self.qk_norm_eps is not None) or self.value_dim != self.head_dim
+        self.wide = not self.prepared and ((self.qk_norm == "projection" and self.qk_norm_eps is not None) or self.value_dim != self.head_dim)
         if self.wide and self.qk_norm == "head" and self.qk_norm_eps is not None:
             raise NotImplementedError("a norm per head together with values of another size than the keys is not supported")
         if self.heads % self.kv_heads:
             raise ValueError(f"{self.heads} query heads are no multiple of {self.kv_heads} KV heads")
         # What the attention kernels refuse is refused here, when the model is built, not in its first step.
-        if not (1 <= self.head_dim <= 256 and 1 <= self.value_dim <= 256):
-            raise ValueError(f"head sizes {self.head_dim} / {self.value_dim} are not supported: the attention kernels take sizes up to 256")
+        limit = 1024 if self.sinks else 256  # what the kernels that know sinks take
+        if not (1 <= self.head_dim <= limit and 1 <= self.value_dim <= limit):
+            raise ValueError(f"head sizes {self.head_dim} / {self.value_dim} are not supported: the attention kernels take sizes up to {limit}")
         if not self.scale > 0:
             raise ValueError(f"the attention scale must be positive, not {self.scale}")
-        generic = self.wide or self.exact_weights or self.keep_first
+        generic = self.wide or self.exact_weights or self.keep_first or self.prepared
         if rt is not None and rt.dtype == torch.bfloat16 and not generic and not (
                 self.head_dim in (64, 128) and self.heads // self.kv_heads <= 16):
             warnings.warn(
@@ -82,7 +103,8 @@ class GQAttention(Mixer):
                 "with up to 16 query heads per KV head", stacklevel=2)
         pos = spec.get("position") or PartSpec("none")
         self.position = part_class("position", pos)(pos, rt)
-        self.qkv = self.o = self.q_norm = self.k_norm = None
+        self.qkv = self.o = self.q_norm = self.k_norm = self.sink = None
+        self.blend = 0.0
 
     @classmethod
     def tensors(cls, spec: PartSpec) -> dict[str, TensorSpec]:
@@ -96,10 +118,15 @@ class GQAttention(Mixer):
             n["v"]: TensorSpec((hkv * dv, h)),
             n["o"]: TensorSpec((h, hq * dv)),
         }
-        if spec.get("qk_norm_eps") is not None:
+        if spec.get("qk_norm_eps") is not None and spec.get("qk_norm_weights", True):
             whole = spec.get("qk_norm", "head") == "projection"
             out[n["q_norm"]] = TensorSpec((hq * d if whole else d,), init="ones")
             out[n["k_norm"]] = TensorSpec((hkv * d if whole else d,), init="ones")
+        if spec.get("sinks", False):
+            out[n["sink"]] = TensorSpec((hq,), init="uniform")
+        if "blend" in (spec.get("names") or {}) or spec.get("value_blend") == "blend":
+            # one number; a layer that does not blend may still carry it, and nothing reads it there
+            out[n["blend"]] = TensorSpec((), init="uniform", optional=spec.get("value_blend") != "blend")
         return out
 
     def bind(self, tensors) -> None:
@@ -109,9 +136,13 @@ class GQAttention(Mixer):
             raise ValueError(f"{p}q/k/v projections are stored in different dtypes")
         self.qkv = torch.cat(parts, dim=0).contiguous()
         self.o = tensors[n["o"]]
-        if self.qk_norm_eps is not None:
+        if self.qk_norm_eps is not None and self.qk_norm_weights:
             self.q_norm = tensors[n["q_norm"]]
             self.k_norm = tensors[n["k_norm"]]
+        if self.sinks:
+            self.sink = tensors[n["sink"]].to(torch.float32).contiguous()
+        if self.value_blend == "blend":
+            self.blend = float(tensors[n["blend"]].to(torch.float32).item())  # one number, read once
 
     def kv_need(self) -> KVNeed:
         return KVNeed.keys_values(self.kv_heads, self.head_dim, self.window, self.value_dim, self.keep_first)
@@ -122,6 +153,8 @@ class GQAttention(Mixer):
         table = rot.table if rot is not None else None
         pairing = rot.pairing if rot is not None else "halves"
         eps = 0.0 if self.qk_norm_eps is None else float(self.qk_norm_eps)
+        if self.prepared:
+            return self._forward_prepared(x, batch, cache, residual, table, pairing, eps)
         if self.wide:
             qkv = ops.linear(x, self.qkv, out_dtype=torch.float32)  # the norms' input is not rounded
             q = ops.qkv_norm_rope_store(qkv, cache.slots if cache.writes else None, self.q_norm, self.k_norm, eps, table,
@@ -155,8 +188,33 @@ class GQAttention(Mixer):
         )
         return ops.linear(out, self.o, accumulate_into=residual, defer=True)
 
+    def _forward_prepared(self, x, batch, cache, residual, table, pairing, eps):
+        ops = self.rt.ops
+        qkv = ops.linear(x, self.qkv, out_dtype=torch.float32)  # what norms and blends read is not rounded
+        v_first = None
+        if self.value_blend is not None:
+            if not cache.writes:
+                raise NotImplementedError("a layer that blends values keeps keys and values of its own")
+            if self.value_blend == "first":
+                # a view of this step's projection: the values as projected, one row per token
+                batch.memo[self.blend_key] = qkv[:, (self.heads + self.kv_heads) * self.head_dim:]
+            else:
+                v_first = batch.memo.get(self.blend_key)
+                if v_first is None:
+                    raise ValueError(f"no earlier layer of the step kept values for {self.blend_key[1]!r}")
+                if v_first.shape[1] != self.kv_heads * self.value_dim:
+                    raise ValueError(f"values of width {self.kv_heads * self.value_dim} cannot be blended with kept values of "
+                                     f"width {v_first.shape[1]}")
+        norm = None if self.qk_norm_eps is None else ("after" if self.qk_norm == "head_rotated" else "before")
+        q = ops.head_prepare_store(qkv, cache.slots if cache.writes else None, norm, self.q_norm, self.k_norm, eps, table, pairing,
+                                   cache.k, cache.v, self.heads, self.kv_heads, self.head_dim, self.value_dim, self.rt.dtype,
+                                   v_first, self.blend)
+        out = ops.paged_attention(q, cache.k, cache.v, cache.block_table, batch, self.heads, self.kv_heads, self.head_dim,
+                                  self.scale, self.window, self.value_dim, sinks=self.sink)
+        return ops.linear(out, self.o, accumulate_into=residual, defer=True)
+
     def parameters_bytes(self) -> int:
-        ts = [self.qkv, self.o] + ([self.q_norm, self.k_norm] if self.q_norm is not None else [])
+        ts = [self.qkv, self.o] + ([self.q_norm, self.k_norm] if self.q_norm is not None else []) + ([self.sink] if self.sink is not None else [])
         return sum(t.numel() * t.element_size() for t in ts)
 
     def flops(self, rows) -> int:

@@ -75,7 +75,10 @@ class OutputNormBlock(Block):
     """``h += norm1(mixer(h)); h += norm2(feed_forward(h))``: the sublayers read the stream itself, and what they put
     out is normed before it joins the stream. Each sublayer adds into a stream of its own that starts at zero; the
     norm's ``add_normed`` folds it into the residual stream. A layer without a feed-forward has no second norm
-    (``ffn_norm`` None); ``spare`` then names norm tensors ``{name: width}`` that a checkpoint may still carry for it."""
+    (``ffn_norm`` None); ``spare`` then names norm tensors ``{name: width}`` that a checkpoint may still carry for it.
+    ``mixer_scale`` / ``ffn_scale`` (optional) name a tensor ``[width]`` each by which the normed output is multiplied
+    element by element before it joins the stream (a layer scale): ``h += scale * norm(sublayer(h))``. It is folded into
+    the norm's weight when the tensors are bound."""
 
     def __init__(self, spec: PartSpec, rt, mixer, feed_forward):
         super().__init__(spec, rt, mixer, feed_forward)
@@ -90,14 +93,21 @@ class OutputNormBlock(Block):
             s = spec.get(key)
             if s is not None:
                 out.update(part_class("norm", s).tensors(s))
+        for key, norm in (("mixer_scale", "mixer_norm"), ("ffn_scale", "ffn_norm")):
+            if spec.get(key) and spec.get(norm) is not None:
+                out[spec[key]] = TensorSpec((int(spec[norm]["width"]),), init="ones")
         for name, width in (spec.get("spare") or {}).items():
             out[name] = TensorSpec((int(width),), optional=True)
         return out
 
     def bind(self, tensors) -> None:
         self.mixer_norm.bind(tensors)
+        if self.spec.get("mixer_scale"):
+            self.mixer_norm.fold_scale(tensors[self.spec["mixer_scale"]])
         if self.ffn_norm is not None:
             self.ffn_norm.bind(tensors)
+            if self.spec.get("ffn_scale"):
+                self.ffn_norm.fold_scale(tensors[self.spec["ffn_scale"]])
 
     def _sublayer(self, run, norm, residual) -> None:
         ops = self.rt.ops

@@ -9,7 +9,14 @@ once; the down projection adds into the residual stream in its epilogue.
 ``<x>_proj.weight``); ``limit`` belongs to the activations that bound their inputs (``swiglu_clamped``).
 ``none`` is the feed-forward of a layer that has none. ``dense_mlp`` (no counterpart in the reference) is
 ``down(act(up(x)))`` without a gate: tensors ``up`` / ``down`` (``names``), the activation in float32 on the float32
-result of the first product, rounded once."""
+result of the first product, rounded once.
+
+``moe_mlp`` (no counterpart in the reference) is a mixture of ``num_experts`` gated feed-forwards of which every token
+runs ``top``: router logits ``router x (+ router_bias)`` in float32, the ``top`` largest chosen (ties: the lower index),
+weights the softmax over the chosen logits alone, the output the weighted sum of the chosen experts' outputs. ``shared``
+(optional) is the ``PartSpec`` of any registered feed-forward that runs for every token and is added. ``names`` maps
+``router``, ``router_bias``, ``expert`` (a pattern with ``{}`` for the expert's number, behind the prefix) and ``gate`` /
+``up`` / ``down`` (behind the expert's own prefix)."""
 
 from __future__ import annotations
 
@@ -17,7 +24,7 @@ import torch
 
 from ..config.spec import PartSpec
 from .base import FeedForward, TensorSpec
-from .registry import register
+from .registry import part_class, register
 
 def _names(spec: PartSpec) -> dict[str, str]:
     p = spec.get("prefix", "")
@@ -110,3 +117,89 @@ class DenseMLP(FeedForward):
 
     def flops(self, rows) -> int:
         return 2 * sum(n for n, _ in rows) * 2 * self.hidden * self.inter
+
+
+def _moe_names(spec: PartSpec) -> dict[str, str]:
+    given = spec.get("names") or {}
+    default = {"router": "router.weight", "router_bias": "router.bias", "expert": "experts.{}.", "gate": "gate_proj.weight",
+               "up": "up_proj.weight", "down": "down_proj.weight"}
+    return {k: given.get(k, d) for k, d in default.items()}
+
+
+@register("feed_forward", "moe_mlp")
+class MixtureMLP(FeedForward):
+    def __init__(self, spec: PartSpec, rt):
+        super().__init__(spec, rt)
+        self.prefix = spec.get("prefix", "")
+        self.hidden = int(spec["hidden_size"])
+        self.inter = int(spec["intermediate_size"])
+        self.num_experts = int(spec["num_experts"])
+        self.top = int(spec["top"])
+        self.activation = spec.get("activation", "silu")
+        self.router_bias = bool(spec.get("router_bias", False))
+        if not 1 <= self.top <= self.num_experts:
+            raise ValueError(f"top {self.top} of {self.num_experts} experts")
+        if rt is not None:
+            ops = rt.ops
+            if self.activation not in ops.ACTIVATIONS or self.activation in ops.ACTIVATIONS_WITH_LIMIT:
+                raise NotImplementedError(f"activation {self.activation!r} is not of the form act(gate) * up")
+            if self.num_experts > ops.MOE_MAX_EXPERTS or self.top > ops.MOE_MAX_TOP:
+                raise ValueError(f"{self.num_experts} experts / top {self.top}: the kernels take up to {ops.MOE_MAX_EXPERTS} "
+                                 f"experts and {ops.MOE_MAX_TOP} choices")
+        self.names = _moe_names(spec)
+        sh = spec.get("shared")
+        self.shared = part_class("feed_forward", sh)(sh, rt) if sh is not None else None
+        self.router = self.bias = self.gate = self.up = self.down = None
+
+    @classmethod
+    def _expert_names(cls, spec: PartSpec, j: int) -> dict[str, str]:
+        n, p = _moe_names(spec), spec.get("prefix", "")
+        return {k: p + n["expert"].format(j) + n[k] for k in ("gate", "up", "down")}
+
+    @classmethod
+    def tensors(cls, spec: PartSpec) -> dict[str, TensorSpec]:
+        n, p = _moe_names(spec), spec.get("prefix", "")
+        h, i, e = int(spec["hidden_size"]), int(spec["intermediate_size"]), int(spec["num_experts"])
+        out = {p + n["router"]: TensorSpec((e, h))}
+        if spec.get("router_bias", False):
+            out[p + n["router_bias"]] = TensorSpec((e,), init="uniform")
+        for j in range(e):
+            en = cls._expert_names(spec, j)
+            out[en["gate"]], out[en["up"]], out[en["down"]] = TensorSpec((i, h)), TensorSpec((i, h)), TensorSpec((h, i))
+        sh = spec.get("shared")
+        if sh is not None:
+            out.update(part_class("feed_forward", sh).tensors(sh))
+        return out
+
+    def bind(self, tensors) -> None:
+        n, p = self.names, self.prefix
+        self.router = tensors[p + n["router"]]
+        self.bias = tensors[p + n["router_bias"]] if self.router_bias else None
+        per = [self._expert_names(self.spec, j) for j in range(self.num_experts)]
+        if len({tensors[en[k]].dtype for en in per for k in en}) != 1:
+            raise ValueError(f"{p}: the experts' projections are stored in different dtypes")
+        # one tensor per projection, [experts, rows, columns]: a kernel finds an expert's weights by its number
+        self.gate, self.up, self.down = (torch.stack([tensors[en[k]] for en in per]).contiguous() for k in ("gate", "up", "down"))
+        if self.shared is not None:
+            self.shared.bind(tensors)
+
+    def forward(self, x, residual):
+        ops = self.rt.ops
+        pending = self.shared.forward(x, residual) if self.shared is not None else None
+        logits = ops.linear(x, self.router, out_dtype=torch.float32)
+        ids, weights = ops.moe_route(logits, self.bias, self.top)
+        xe = ops.cast(x, self.gate.dtype)  # experts stored in 32-bit compute in 32-bit
+        ops.moe_experts(xe, ids, weights, self.gate, self.up, self.down, self.activation, residual)
+        return pending
+
+    def parameters_bytes(self) -> int:
+        """What one token reads: the router, its ``top`` experts and the shared expert (a step of several tokens reads up
+        to ``top`` experts more per token)."""
+        per_expert = sum(t[0].numel() * t.element_size() for t in (self.gate, self.up, self.down))
+        own = self.router.numel() * self.router.element_size() + self.top * per_expert
+        return own + (self.shared.parameters_bytes() if self.shared is not None else 0)
+
+    def flops(self, rows) -> int:
+        tokens = sum(n for n, _ in rows)
+        own = 2 * tokens * self.hidden * self.num_experts + 2 * tokens * self.top * 3 * self.hidden * self.inter
+        return own + (self.shared.flops(rows) if self.shared is not None else 0)

@@ -4,7 +4,8 @@ model dtype before the weight product; here the whole expression is evaluated in
 rounded once, which is what its fused operators do (miniserve/model/fused.py:188-194).
 
 ``offset`` (optional, no counterpart in the reference): the stored weight lies around zero and the norm multiplies by
-``offset + w`` (``offset = 1``: the "one plus weight" form). The sum is formed once, in float32, when the weight is bound."""
+``offset + w`` (``offset = 1``: the "one plus weight" form). The sum is formed once, in float32, when the weight is bound.
+``fold_scale`` lets a block hang a scale per channel behind the norm (a layer scale) at no cost per step."""
 
 from __future__ import annotations
 
@@ -33,6 +34,11 @@ class RMSNorm(Norm):
         self.weight = tensors[self.spec["tensor"]]
         if self.offset:
             self.weight = (self.weight.to(torch.float32) + self.offset).contiguous()
+
+    def fold_scale(self, scale) -> None:
+        """Multiply what the norm puts out by ``scale [width]``, element by element: the product with the weight is
+        formed once, in float32 (two bfloat16 numbers multiply exactly there), and takes the weight's place."""
+        self.weight = (self.weight.to(torch.float32) * scale.to(torch.float32)).contiguous()
 
     def forward(self, x, rows=None, add=None):
         """``x``: float32 ``[T, width]``; ``rows``: optional int32 row indices to normalise (the
