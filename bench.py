@@ -25,7 +25,7 @@ with its share of the roofline), ``measured_peaks`` (what this box gives a strea
 and the engine's bfloat16 product) and ``sidecar`` (device, clocks and power while the headline point
 ran, versions, commit, the engine's effective configuration).
 
-``--design kakunex`` (or ``fimolix``) measures something else and leaves the above as it is: prefill and decode
+``--design kakunex`` (or ``fimolix``, ``reselorn``) measures something else and leaves the above as it is: prefill and decode
 throughput of that architecture beside Qwen3 models of equal size (``miniserve_amd/measurement/designs.py``), one JSON line.
 
 Peaks: MI355X's published 8 TB/s HBM and 2.5 PFLOP/s dense bf16 (157.3 TFLOP/s float32).
@@ -74,7 +74,7 @@ def main() -> int:
     ap.add_argument("--prefill-tokens", type=int, default=2048, help="tokens of the timed prefill step")
     ap.add_argument("--prefill-cached", type=int, default=0,
                     help="tokens of the same sequence already in the cache when the timed step runs (fed untimed, 2,048 a step)")
-    ap.add_argument("--design", choices=("kakunex", "fimolix"), default=None,
+    ap.add_argument("--design", choices=("kakunex", "fimolix", "reselorn"), default=None,
                     help="instead of the workload above: prefill and decode of this architecture beside Qwen3 of equal size")
     ap.add_argument("--shapes", default=None, help="with --design: the shapes to run, with commas between them (default: all)")
     args = ap.parse_args()

@@ -1,6 +1,6 @@
 """Prefill and decode throughput of one architecture beside another of equal size: random weights, layers of the
-sizes real models have, the same step function for both. ``bench.py --design kakunex`` (or ``fimolix``) prints what
-this returns.
+sizes real models have, the same step function for both. ``bench.py --design kakunex`` (or ``fimolix``, ``reselorn``)
+prints what this returns.
 
 A *shape* fixes what the two share: width, query and key/value heads of 128 elements, feed-forward width, window,
 layers, vocabulary. The Kakunex model of a shape repeats (parallel, parallel, parallel, mlstm): window attention that
@@ -12,7 +12,12 @@ The Fimolix model of a shape repeats (latent attention, differential attention, 
 attention that reads the first one's cache). Its differential attention has half the shape's heads, each with two maps
 of 128 and values of 256, so that its four projections have the sizes of the Qwen3 layer's; convolutions of 4 taps. Its
 latent attention has the shape's query heads with 128 plain and 64 rotated elements, values of 128 and a latent of 512
-per token, inside the shape's window."""
+per token, inside the shape's window.
+
+The Reselorn model of a shape has the shape's heads of 128 elements (half of them rotated, slowed frequencies), a sink
+per head, the shape's window and blended values in every layer; its first layer has the shape's dense feed-forward, the
+others a mixture of 32 experts of an eighth of that width, of which a token runs 4, beside a shared expert of half the
+width: a token multiplies as much as in the Qwen3 layer, the weights are 4.5 times the layer's."""
 
 from __future__ import annotations
 
@@ -72,7 +77,20 @@ def fimolix_config(s: dict) -> dict:
     return {"architecture": "Fimolix", "vocab": s["vocab"], "width": s["width"], "norm": {"eps": 1e-6}, "layers": layers}
 
 
-DESIGNS = {"kakunex": kakunex_config, "fimolix": fimolix_config, "qwen3": qwen3_config}
+EXPERTS, CHOSEN = 32, 4
+
+
+def reselorn_config(s: dict) -> dict:
+    mixer = {"heads": s["heads"], "kv_heads": s["kv_heads"], "dim": HEAD, "vdim": HEAD, "scale": HEAD ** -0.5, "v_mix": True,
+             "rot": {"base": 1.5e5, "dims": HEAD // 2, "scaling": {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}},
+             "mask": {"size": s["window"]}}
+    mixture = {"kind": "moe", "router": {"experts": EXPERTS, "top": CHOSEN}, "expert": {"ff": s["ff"] // 8}, "shared": {"ff": s["ff"] // 2}}
+    layers = [{"type": "attention", "mixer": dict(mixer), "mlp": {"kind": "dense", "ff": s["ff"]} if i == 0 else mixture}
+              for i in range(s["layers"])]
+    return {"architecture": "Reselorn", "vocab": s["vocab"], "width": s["width"], "norm": {"eps": 1e-6}, "layers": layers}
+
+
+DESIGNS = {"kakunex": kakunex_config, "fimolix": fimolix_config, "reselorn": reselorn_config, "qwen3": qwen3_config}
 
 
 def measure(config: dict, dtype: str, prefill_tokens: int, batch: int, context: int, steps: int, warmup: int, say=lambda m: None) -> dict:

@@ -74,7 +74,8 @@ def _turn_ramp(inv_freq: torch.Tensor, scaling: dict, theta: float) -> torch.Ten
     lo = max(math.floor(index_of(fast)), 0)
     hi = min(math.ceil(index_of(slow)), dim - 1)
     out = []
-    for j, f in enumerate(inv_freq.to(torch.float64).tolist()):
+    for j in range(dim // 2):
+        f = theta ** (-2.0 * j / dim)  # in double precision: the blend is rounded to float32 once
         r = min(max((j - lo) / max(hi - lo, 0.001), 0.0), 1.0)
         out.append(r * f / factor + (1 - r) * f)
     return torch.tensor(out, dtype=torch.float64).to(torch.float32)
