@@ -215,6 +215,164 @@ __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(
   }
 }
 
+// The same two products for steps with many pairs per expert (K a multiple of 64, rows 16-byte aligned): tiles of BM pairs
+// x 128 weight rows, K in slabs of 64 that go straight into LDS (global_load_lds, 16 bytes a lane) in a ring of two
+// stages, one barrier per slab, two blocks per CU. A load instruction of a wave fills 1 KB of LDS in lane order, that is
+// 8 tile rows of 128 bytes; the 16-byte chunk c of tile row R lands in slot c ^ ((R >> 1) & 7) of its row, so that a
+// fragment read (16 rows, one chunk column) touches every bank once. The weight rows are the matrix instruction's first
+// operand and the pairs its second: a lane ends up with four consecutive columns of one pair.
+//   GATED: the tile's weight rows are blocks of 16 gate rows and 16 up rows in turn (64 columns of h a block), so that a
+//          lane's fragments 2 i and 2 i + 1 are gate and up of the same four outputs.
+// Pairs past the tile's count read the tile's last pair, weight rows past N the last row: their results are not stored.
+// Every output element is the same chain of products over k as in the kernel above, whatever the tile.
+template <int N_> __device__ __forceinline__ void moe_wait_loads() {
+  __builtin_amdgcn_s_waitcnt((N_ & 15) | ((N_ >> 4) << 14) | (7 << 4) | (15 << 8));  // vmcnt alone
+}
+
+template <bool GATED, int BM, int WR, int WC>
+__global__ __launch_bounds__(256, 2) void moe_gemm_bf16_lds_kernel(
+    const bf16* __restrict__ a, int lda, const bf16* __restrict__ w1, const bf16* __restrict__ w2, void* __restrict__ out,
+    const int* __restrict__ order, const int* __restrict__ tile_expert, const int* __restrict__ tile_start,
+    const int* __restrict__ tile_count, const float* __restrict__ pair_weight, int top, int N, int K, int act) {
+  static_assert(WR * WC == 4, "four waves a block");
+  constexpr int BN = 128, KS = 64, STAGES = 2;
+  constexpr int WM = BM / WR, WN = BN / WC, FM = WM / 16, FN = WN / 16;
+  constexpr int ROW_BYTES = KS * 2, CPR = 8, RPI = 8;
+  constexpr int XI = BM / (4 * RPI), WI = BN / (4 * RPI);
+  constexpr int STAGE_BYTES = (BM + BN) * ROW_BYTES;
+  static_assert(!GATED || FN % 2 == 0, "gate and up fragments come in pairs");
+  extern __shared__ __attribute__((aligned(1024))) unsigned char moe_lds[];
+  const int tile = blockIdx.y;
+  const int count = tile_count[tile];
+  if (count == 0) return;
+  const int e = tile_expert[tile], start = tile_start[tile];
+  const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
+  const int r = lane % 16, g = lane / 16;
+  const int n0 = blockIdx.x * (GATED ? BN / 2 : BN);  // first output column of the tile
+  const int wm = (wave / WC) * WM, wn = (wave % WC) * WN;
+  const int slabs = K / KS;
+
+  const int lrow = lane / CPR, lslot = lane % CPR;
+  const bf16* xsrc[XI];
+  const bf16* wsrc[WI];
+#pragma unroll
+  for (int j = 0; j < XI; ++j) {
+    const int R = (wave * XI + j) * RPI + lrow;
+    const int place = start + min(R, count - 1);
+    xsrc[j] = a + (size_t)(GATED ? order[place] / top : place) * lda + ((lslot ^ ((R >> 1) & (CPR - 1))) * 8);
+  }
+#pragma unroll
+  for (int j = 0; j < WI; ++j) {
+    const int R = (wave * WI + j) * RPI + lrow;
+    const int chunk = (lslot ^ ((R >> 1) & (CPR - 1))) * 8;
+    if (GATED) {
+      const int n = min(n0 + (R / 32) * 16 + R % 16, N - 1);
+      wsrc[j] = (((R / 16) & 1) ? w2 : w1) + ((size_t)e * N + n) * K + chunk;
+    } else {
+      wsrc[j] = w1 + ((size_t)e * N + min(n0 + R, N - 1)) * K + chunk;
+    }
+  }
+  auto issue = [&](int slab) __attribute__((always_inline)) {
+    unsigned char* stage = moe_lds + (slab % STAGES) * STAGE_BYTES;
+#pragma unroll
+    for (int j = 0; j < XI; ++j)
+      __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1)))*)(xsrc[j] + (size_t)slab * KS),
+                                       (void __attribute__((address_space(3)))*)(stage + (wave * XI + j) * 1024), 16, 0, 0);
+#pragma unroll
+    for (int j = 0; j < WI; ++j)
+      __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1)))*)(wsrc[j] + (size_t)slab * KS),
+                                       (void __attribute__((address_space(3)))*)(stage + BM * ROW_BYTES + (wave * WI + j) * 1024),
+                                       16, 0, 0);
+  };
+
+  moe_floatx4 acc[FN][FM];
+#pragma unroll
+  for (int i = 0; i < FN; ++i)
+#pragma unroll
+    for (int j = 0; j < FM; ++j) acc[i][j] = moe_floatx4{0.f, 0.f, 0.f, 0.f};
+  const int sw = (r >> 1) & (CPR - 1);
+  const int x_off = (wm + r) * ROW_BYTES, w_off = BM * ROW_BYTES + (wn + r) * ROW_BYTES;
+
+  issue(0);
+  for (int k = 0; k < slabs; ++k) {
+    moe_wait_loads<0>();
+    __syncthreads();  // slab k has landed for every wave, and every wave is done with slab k - 1
+    if (k + 1 < slabs) issue(k + 1);
+    const unsigned char* stage = moe_lds + (k % STAGES) * STAGE_BYTES;
+    moe_bf16x8 wf[2][FN], xf[2][FM];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const int slot = ((t * 4 + g) ^ sw) * 16;
+#pragma unroll
+      for (int i = 0; i < FN; ++i) wf[t][i] = *reinterpret_cast<const moe_bf16x8*>(stage + w_off + i * 16 * ROW_BYTES + slot);
+#pragma unroll
+      for (int j = 0; j < FM; ++j) xf[t][j] = *reinterpret_cast<const moe_bf16x8*>(stage + x_off + j * 16 * ROW_BYTES + slot);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int i = 0; i < FN; ++i)
+#pragma unroll
+        for (int j = 0; j < FM; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[t][i], xf[t][j], acc[i][j], 0, 0, 0);
+  }
+
+  const bool vec = N % 4 == 0;
+#pragma unroll
+  for (int j = 0; j < FM; ++j) {
+    const int m = wm + j * 16 + r;
+    if (m >= count) continue;
+    if (GATED) {
+      bf16* o = (bf16*)out + (size_t)(start + m) * N;
+#pragma unroll
+      for (int i = 0; i + 1 < FN; i += 2) {
+        const int col = n0 + wn / 2 + (i / 2) * 16 + g * 4;
+        union { uint2 u; bf16 v[4]; } q;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) q.v[c] = static_cast<bf16>(gated_value(acc[i][j][c], acc[i + 1][j][c], act, 0.f));
+        if (vec && col + 3 < N) *reinterpret_cast<uint2*>(o + col) = q.u;
+        else
+#pragma unroll
+          for (int c = 0; c < 4; ++c)
+            if (col + c < N) o[col + c] = q.v[c];
+      }
+    } else {
+      const int pair = order[start + m];
+      const float pw = pair_weight[pair];
+      float* o = (float*)out + (size_t)pair * N;
+#pragma unroll
+      for (int i = 0; i < FN; ++i) {
+        const int col = n0 + wn + i * 16 + g * 4;
+        if (vec && col + 3 < N) *reinterpret_cast<float4*>(o + col) = make_float4(acc[i][j][0] * pw, acc[i][j][1] * pw, acc[i][j][2] * pw, acc[i][j][3] * pw);
+        else
+#pragma unroll
+          for (int c = 0; c < 4; ++c)
+            if (col + c < N) o[col + c] = acc[i][j][c] * pw;
+      }
+    }
+  }
+}
+
+template <bool GATED, int BM, int WR, int WC>
+static int moe_launch_lds(const void* a, int lda, const void* w1, const void* w2, void* out, const int* order, const int* tile_expert,
+                          const int* tile_start, const int* tile_count, const float* pair_weight, int max_tiles, int top, int N,
+                          int K, int act, hipStream_t st) {
+  constexpr int lds_bytes = 2 * (BM + 128) * 128;
+  static bool ready = false;  // more than 48 KB of LDS is asked for once per kernel
+  if (!ready) {
+    if (hipFuncSetAttribute((const void*)moe_gemm_bf16_lds_kernel<GATED, BM, WR, WC>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            lds_bytes) != hipSuccess)
+      return MS_LAUNCH_FAILED;
+    ready = true;
+  }
+  const int cols = GATED ? 64 : 128;
+  const dim3 grid((N + cols - 1) / cols, max_tiles);
+  if (grid.y > 65535) return MS_BAD_ARG;
+  moe_gemm_bf16_lds_kernel<GATED, BM, WR, WC><<<grid, 256, lds_bytes, st>>>((const bf16*)a, lda, (const bf16*)w1, (const bf16*)w2, out, order,
+                                                                           tile_expert, tile_start, tile_count, pair_weight, top, N, K, act);
+  return launch_status();
+}
+
 // The same two products in true float32 on the vector units: 64 x 64 tiles through LDS, every output element one chain of
 // fused multiply-adds over k in ascending order.
 template <bool GATED>
@@ -294,7 +452,8 @@ __global__ __launch_bounds__(256) void moe_gemm_f32_kernel(
 }
 
 // a: the rows ([tokens, lda] for the gated product, [P, lda] sorted places for the other); w1 (and w2, gated): [E, N, K];
-// out: h [P, N] (gated, the compute type) or y [P, N] float32. tile_rows: 16 or 64 in bfloat16, 64 in float32.
+// out: h [P, N] (gated, the compute type) or y [P, N] float32. tile_rows: 16, 64 or 128 in bfloat16 (128: K a multiple of
+// 64 and 16-byte aligned rows), 64 in float32.
 extern "C" int ms_moe_gemm(const void* a, int lda, const void* w1, const void* w2, void* out, int is_bf16, int gated,
                            const int* order, const int* tile_expert, const int* tile_start, const int* tile_count,
                            const float* pair_weight, int max_tiles, int top, int N, int K, int tile_rows, int act, hipStream_t st) {
@@ -304,7 +463,15 @@ extern "C" int ms_moe_gemm(const void* a, int lda, const void* w1, const void* w
       act < 0 || act >= MS_ACT_COUNT)
     return MS_BAD_ARG;
   if (is_bf16) {
-    if (tile_rows != 16 && tile_rows != 64) return MS_BAD_ARG;
+    if (tile_rows != 16 && tile_rows != 64 && tile_rows != 128) return MS_BAD_ARG;
+    const bool rows16 = (size_t)a % 16 == 0 && (size_t)w1 % 16 == 0 && (!gated || (size_t)w2 % 16 == 0) && lda % 8 == 0;
+    if (tile_rows >= 64 && K % 64 == 0 && rows16 && (gated || (size_t)out % 16 == 0)) {
+#define MOE_LDS(G, BM, WR, WC) moe_launch_lds<G, BM, WR, WC>(a, lda, w1, w2, out, order, tile_expert, tile_start, tile_count, pair_weight, max_tiles, top, N, K, act, st)
+      if (tile_rows == 128) return gated ? MOE_LDS(true, 128, 2, 2) : MOE_LDS(false, 128, 2, 2);
+      return gated ? MOE_LDS(true, 64, 1, 4) : MOE_LDS(false, 64, 1, 4);
+#undef MOE_LDS
+    }
+    if (tile_rows == 128) return MS_UNSUPPORTED;  // the caller plans tiles of 128 only where the kernel above takes them
     const int cols = tile_rows == 64 ? 64 : 256;
     const dim3 grid(max_tiles, (N + cols - 1) / cols);
     if (grid.y > 65535) return MS_BAD_ARG;

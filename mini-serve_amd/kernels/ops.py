@@ -466,6 +466,7 @@ def add_pending(residual: torch.Tensor, pending: SplitSum | None) -> None:
 MOE_MAX_EXPERTS = 512  # MOE_MAX_EXPERTS in csrc/moe.hip
 MOE_MAX_TOP = 64
 MOE_SMALL_TILE_PAIRS = 16  # (token, expert) pairs per expert, on average, up to which a step runs 16-pair tiles
+MOE_LARGE_TILE_PAIRS = 128  # ... and from which it runs 128-pair tiles (widths that are multiples of 64)
 
 
 def moe_route(logits: torch.Tensor, bias: torch.Tensor | None, top: int):
@@ -521,6 +522,9 @@ def moe_experts(x: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, gate:
     pairs = t * top
     bf = x.dtype == BF16
     tile_rows = 16 if bf and pairs <= MOE_SMALL_TILE_PAIRS * e else 64
+    if bf and pairs >= MOE_LARGE_TILE_PAIRS * e and width % 64 == 0 and f % 64 == 0 and not any(
+            t.data_ptr() % 16 for t in (x, gate, up, down)):
+        tile_rows = 128  # both products then run tiles of 128 pairs staged through LDS
     max_tiles = -(-pairs // tile_rows) + min(e, pairs)
     dev = x.device
     order = torch.empty((pairs,), dtype=I32, device=dev)
