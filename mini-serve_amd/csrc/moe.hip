@@ -126,9 +126,10 @@ extern "C" int ms_moe_plan(const int* ids, int P, int E, int tile_rows, int max_
 
 // ---------------------------------------------------------------------------------------------
 // The experts' products on the matrix cores (bfloat16 operands, float32 sums, v_mfma_f32_16x16x32_bf16), operands
-// straight from memory, 16 bytes a lane. A wave owns 16 pairs x 64 columns; a block's four waves split a tile of 64 pairs
-// by rows (64 columns a block), a tile of 16 pairs by columns (256 columns a block: steps of few tokens, where every
-// chosen expert has a tile of its own and its weights are streamed once).
+// straight from memory, 16 bytes a lane. A wave owns 16 pairs x 16 NT columns; a block's four waves split a tile of 64
+// pairs by rows (NT = 4: 64 columns a block), a tile of 16 pairs by columns (64 NT columns a block: steps of few tokens,
+// where every chosen expert has a tile of its own and its weights are streamed once; the fewer tiles the step can have,
+// the narrower the waves' runs of columns, so that the chip still gets waves enough to stream with).
 //   GATED: rows are x[token of the pair] (K = the model's width), two weights per expert, gate and up [E, N, K]; the result
 //          act(gate) * up goes to h[sorted place][N] in the compute type.
 //   else:  rows are h[sorted place] (K = the experts' width), one weight per expert [E, N, K]; the result times the pair's
@@ -151,7 +152,7 @@ template <bool ALIGNED> __device__ __forceinline__ moe_bf16x8 moe_load(const bf1
   return x.v;
 }
 
-template <bool GATED, bool ALIGNED>
+template <bool GATED, bool ALIGNED, int NT>
 __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(
     const bf16* __restrict__ a, int lda, const bf16* __restrict__ w1, const bf16* __restrict__ w2, void* __restrict__ out,
     const int* __restrict__ order, const int* __restrict__ tile_expert, const int* __restrict__ tile_start,
@@ -161,36 +162,37 @@ __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(
   const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE, l16 = lane % 16, grp = lane / 16;
   const bool by_rows = tile_rows == 64;
   const int m0 = by_rows ? wave * 16 : 0;
-  const int n0 = by_rows ? blockIdx.y * 64 : blockIdx.y * 256 + wave * 64;
+  const int n0 = by_rows ? blockIdx.y * (16 * NT) : (blockIdx.y * 4 + wave) * (16 * NT);
   if (m0 >= count || n0 >= N) return;
   const int e = tile_expert[blockIdx.x], start = tile_start[blockIdx.x];
   const bool row_ok = m0 + l16 < count;
   const int place = start + m0 + (row_ok ? l16 : 0);
   const bf16* ap = a + (size_t)(GATED ? order[place] / top : place) * lda;
-  const bf16* wp1[4];
-  const bf16* wp2[4];
-  bool col_ok[4];
+  const bf16* wp1[NT];
+  const bf16* wp2[NT];
+  bool col_ok[NT];
 #pragma unroll
-  for (int nt = 0; nt < 4; ++nt) {
+  for (int nt = 0; nt < NT; ++nt) {
     col_ok[nt] = n0 + nt * 16 + l16 < N;
     const size_t at = ((size_t)e * N + (col_ok[nt] ? n0 + nt * 16 + l16 : 0)) * K;
     wp1[nt] = w1 + at;
     wp2[nt] = GATED ? w2 + at : nullptr;
   }
-  moe_floatx4 acc1[4], acc2[4];
+  moe_floatx4 acc1[NT], acc2[NT];
 #pragma unroll
-  for (int nt = 0; nt < 4; ++nt) acc1[nt] = acc2[nt] = moe_floatx4{0.f, 0.f, 0.f, 0.f};
+  for (int nt = 0; nt < NT; ++nt) acc1[nt] = acc2[nt] = moe_floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll(4 / NT)
   for (int k0 = 0; k0 < K; k0 += 32) {
     const int kk = k0 + grp * 8;  // the lane's eight elements of this step
     const moe_bf16x8 av = moe_load<ALIGNED>(ap, kk, K, row_ok);
-    moe_bf16x8 b1[4], b2[4];
+    moe_bf16x8 b1[NT], b2[NT];
 #pragma unroll
-    for (int nt = 0; nt < 4; ++nt) {
+    for (int nt = 0; nt < NT; ++nt) {
       b1[nt] = moe_load<ALIGNED>(wp1[nt], kk, K, col_ok[nt]);
       if (GATED) b2[nt] = moe_load<ALIGNED>(wp2[nt], kk, K, col_ok[nt]);
     }
 #pragma unroll
-    for (int nt = 0; nt < 4; ++nt) {
+    for (int nt = 0; nt < NT; ++nt) {
       acc1[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, b1[nt], acc1[nt], 0, 0, 0);
       if (GATED) acc2[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, b2[nt], acc2[nt], 0, 0, 0);
     }
@@ -202,14 +204,14 @@ __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(
     if (GATED) {
       bf16* o = (bf16*)out + (size_t)(start + m) * N + n0 + l16;
 #pragma unroll
-      for (int nt = 0; nt < 4; ++nt)
+      for (int nt = 0; nt < NT; ++nt)
         if (col_ok[nt]) o[nt * 16] = static_cast<bf16>(gated_value(acc1[nt][r], acc2[nt][r], act, 0.f));
     } else {
       const int pair = order[start + m];
       const float pw = pair_weight[pair];
       float* o = (float*)out + (size_t)pair * N + n0 + l16;
 #pragma unroll
-      for (int nt = 0; nt < 4; ++nt)
+      for (int nt = 0; nt < NT; ++nt)
         if (col_ok[nt]) o[nt * 16] = acc1[nt][r] * pw;
     }
   }
@@ -472,13 +474,22 @@ extern "C" int ms_moe_gemm(const void* a, int lda, const void* w1, const void* w
 #undef MOE_LDS
     }
     if (tile_rows == 128) return MS_UNSUPPORTED;  // the caller plans tiles of 128 only where the kernel above takes them
-    const int cols = tile_rows == 64 ? 64 : 256;
+    // 16-pair tiles: min(E, pairs) of them at most are in use, each times the column blocks; the narrowest run of columns
+    // with which that is under four blocks a CU.
+    int nt = 4;
+    if (tile_rows == 16) {
+      const long busy = max_tiles / 2 + 1;  // about half of the launched tiles hold pairs
+      while (nt > 1 && busy * ((N + 64 * nt - 1) / (64 * nt)) < 1024) nt /= 2;
+    }
+    const int cols = tile_rows == 64 ? 64 : 64 * nt;
     const dim3 grid(max_tiles, (N + cols - 1) / cols);
     if (grid.y > 65535) return MS_BAD_ARG;
     const bool aligned = K % 8 == 0 && lda % 8 == 0 && (size_t)a % 16 == 0 && (size_t)w1 % 16 == 0 && (!gated || (size_t)w2 % 16 == 0);
-#define MOE(G, A) moe_gemm_bf16_kernel<G, A><<<grid, 256, 0, st>>>((const bf16*)a, lda, (const bf16*)w1, (const bf16*)w2, out, order, tile_expert, tile_start, tile_count, pair_weight, top, N, K, tile_rows, act)
-    if (gated) { if (aligned) MOE(true, true); else MOE(true, false); }
-    else { if (aligned) MOE(false, true); else MOE(false, false); }
+#define MOE(G, A, T) moe_gemm_bf16_kernel<G, A, T><<<grid, 256, 0, st>>>((const bf16*)a, lda, (const bf16*)w1, (const bf16*)w2, out, order, tile_expert, tile_start, tile_count, pair_weight, top, N, K, tile_rows, act)
+#define MOE_NT(G, A) do { if (nt == 4) MOE(G, A, 4); else if (nt == 2) MOE(G, A, 2); else MOE(G, A, 1); } while (0)
+    if (gated) { if (aligned) MOE_NT(true, true); else MOE_NT(true, false); }
+    else { if (aligned) MOE_NT(false, true); else MOE_NT(false, false); }
+#undef MOE_NT
 #undef MOE
   } else {
     if (tile_rows != 64) return MS_BAD_ARG;
