@@ -169,15 +169,18 @@ extern "C" int ms_normed_mean_add(float* residual, const float* const* streams, 
   return launch_status();
 }
 
-// residual += rmsnorm(stream + pending) * w for one stream whose last matrix product left partial sums (`splits` slices
-// `stride` floats apart, added in ascending order): the sums are formed inside the norm instead of being written out by a
-// kernel of their own. A block of 1,024 threads per row; a thread keeps the sums of its first eight elements in registers
-// between the mean of squares and the result (rows up to 8,192 wide are summed once; what lies beyond is summed again).
-// stream may be nullptr (zero).
+// residual += rmsnorm(stream + pending) * w for one stream whose last matrix product may have left partial sums (`splits`
+// slices `stride` floats apart, added in ascending order; parts may be nullptr): the sums are formed inside the norm
+// instead of being written out by a kernel of their own. A block of 1,024 threads per row; a thread keeps the sums of its
+// first eight elements in registers between the mean of squares and the result (rows up to 8,192 wide are summed once;
+// what lies beyond is summed again). stream may be nullptr (zero). What the next reader of the residual would otherwise
+// launch kernels for can ride along: `next` (bfloat16, nullable) receives the new residual rounded, and with `clear` the
+// stream is left zero for the next sublayer to add into.
 template <typename TW>
-__global__ __launch_bounds__(1024) void normed_add_pending_kernel(float* __restrict__ residual, const float* __restrict__ stream,
+__global__ __launch_bounds__(1024) void normed_add_pending_kernel(float* __restrict__ residual, float* __restrict__ stream,
                                                                   const float* __restrict__ parts, int splits, size_t stride,
-                                                                  const TW* __restrict__ w, int width, float eps) {
+                                                                  const TW* __restrict__ w, int width, float eps,
+                                                                  bf16* __restrict__ next, int clear) {
   constexpr int NT = 1024, KEPT = 8;
   __shared__ float red[NT / WAVE];
   const size_t row = (size_t)blockIdx.x * width;
@@ -186,31 +189,41 @@ __global__ __launch_bounds__(1024) void normed_add_pending_kernel(float* __restr
 #pragma unroll
   for (int i = 0; i < KEPT; ++i) {
     const int e = threadIdx.x + i * NT;
-    kept[i] = e < width ? (stream ? stream[row + e] : 0.f) + sum_splits(parts + row + e, splits, stride) : 0.f;
+    kept[i] = e < width ? (stream ? stream[row + e] : 0.f) + (parts ? sum_splits(parts + row + e, splits, stride) : 0.f) : 0.f;
     ss += kept[i] * kept[i];
   }
   for (int e = threadIdx.x + KEPT * NT; e < width; e += NT) {
-    const float v = (stream ? stream[row + e] : 0.f) + sum_splits(parts + row + e, splits, stride);
+    const float v = (stream ? stream[row + e] : 0.f) + (parts ? sum_splits(parts + row + e, splits, stride) : 0.f);
     ss += v * v;
   }
   const float rstd = 1.f / sqrtf(block_sum<NT>(ss, red) / (float)width + eps);
 #pragma unroll
   for (int i = 0; i < KEPT; ++i) {
     const int e = threadIdx.x + i * NT;
-    if (e < width) residual[row + e] += kept[i] * rstd * to_f32(w[e]);
+    if (e < width) {
+      const float r = residual[row + e] + kept[i] * rstd * to_f32(w[e]);
+      residual[row + e] = r;
+      if (next) next[row + e] = static_cast<bf16>(r);
+      if (clear && stream) stream[row + e] = 0.f;
+    }
   }
   for (int e = threadIdx.x + KEPT * NT; e < width; e += NT) {
-    const float v = (stream ? stream[row + e] : 0.f) + sum_splits(parts + row + e, splits, stride);
-    residual[row + e] += v * rstd * to_f32(w[e]);
+    const float v = (stream ? stream[row + e] : 0.f) + (parts ? sum_splits(parts + row + e, splits, stride) : 0.f);
+    const float r = residual[row + e] + v * rstd * to_f32(w[e]);
+    residual[row + e] = r;
+    if (next) next[row + e] = static_cast<bf16>(r);
+    if (clear && stream) stream[row + e] = 0.f;
   }
 }
 
-extern "C" int ms_normed_add_pending(float* residual, const float* stream, const float* parts, int splits, long long stride,
-                                     const void* w, int w_is_bf16, int tokens, int width, float eps, hipStream_t st) {
+extern "C" int ms_normed_add_pending(float* residual, float* stream, const float* parts, int splits, long long stride,
+                                     const void* w, int w_is_bf16, int tokens, int width, float eps, void* next_bf16, int clear,
+                                     hipStream_t st) {
   if (tokens <= 0) return MS_OK;
-  if (width <= 0 || splits < 1 || stride < (long long)tokens * width || parts == nullptr || !(eps >= 0.f)) return MS_BAD_ARG;
-  if (w_is_bf16) normed_add_pending_kernel<bf16><<<tokens, 1024, 0, st>>>(residual, stream, parts, splits, (size_t)stride, (const bf16*)w, width, eps);
-  else normed_add_pending_kernel<float><<<tokens, 1024, 0, st>>>(residual, stream, parts, splits, (size_t)stride, (const float*)w, width, eps);
+  if (width <= 0 || (parts == nullptr && stream == nullptr) || !(eps >= 0.f)) return MS_BAD_ARG;
+  if (parts != nullptr && (splits < 1 || stride < (long long)tokens * width)) return MS_BAD_ARG;
+  if (w_is_bf16) normed_add_pending_kernel<bf16><<<tokens, 1024, 0, st>>>(residual, stream, parts, splits, (size_t)stride, (const bf16*)w, width, eps, (bf16*)next_bf16, clear);
+  else normed_add_pending_kernel<float><<<tokens, 1024, 0, st>>>(residual, stream, parts, splits, (size_t)stride, (const float*)w, width, eps, (bf16*)next_bf16, clear);
   return launch_status();
 }
 

@@ -29,7 +29,8 @@ _SIGNATURES = {
     "ms_layernorm": [_c_void, _c_void, _c_void, _c_int, _c_void, _c_int, _c_void, _c_int, _c_int, _c_float, _c_void],
     "ms_group_rmsnorm_gate": [_c_void, _c_void, _c_int, _c_void, _c_int, _c_void, _c_int, _c_int, _c_int, _c_int, _c_float, _c_void],
     "ms_normed_mean_add": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _c_void],
-    "ms_normed_add_pending": [_c_void, _c_void, _c_void, _c_int, _c_ll, _c_void, _c_int, _c_int, _c_int, _c_float, _c_void],
+    "ms_normed_add_pending": [_c_void, _c_void, _c_void, _c_int, _c_ll, _c_void, _c_int, _c_int, _c_int, _c_float, _c_void, _c_int,
+                              _c_void],
     "ms_scale": [_c_void, _c_ll, _c_float, _c_void],
     "ms_qkv_norm_rope_store": [_c_void, _c_int, _c_void, _c_int, _c_void, _c_void, _c_void, _c_int, _c_float, _c_void, _c_int, _c_int,
                                _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
@@ -1138,25 +1139,34 @@ def normed_mean_add(residual: torch.Tensor, streams, weights, eps: float, coef: 
                                         residual.shape[1], float(eps), float(coef), _stream()), "normed_mean_add")
 
 
-def normed_add(residual: torch.Tensor, stream: torch.Tensor | None, weight: torch.Tensor, eps: float, pending: SplitSum | None = None) -> None:
+def normed_add(residual: torch.Tensor, stream: torch.Tensor | None, weight: torch.Tensor, eps: float, pending: SplitSum | None = None,
+               next_out: torch.Tensor | None = None, clear: bool = False) -> None:
     """``residual += rmsnorm(stream + pending) * weight`` row by row: one float32 stream of the residual's shape (None:
-    zero) and the partial sums its last matrix product may have left (summed inside the kernel, no kernel of their own)."""
-    if pending is None:
-        if stream is None:
-            raise ValueError("neither a stream nor a pending sum")
+    zero) and the partial sums its last matrix product may have left (summed inside the kernel, no kernel of their own).
+    ``next_out`` (bfloat16, the residual's shape) receives the new residual rounded, for the next reader that wants it in
+    16 bits; with ``clear`` the stream is left zero."""
+    if pending is None and stream is None:
+        raise ValueError("neither a stream nor a pending sum")
+    if pending is None and next_out is None and not clear:
         return normed_mean_add(residual, [stream], [weight], eps, 1.0)
     _dev(residual, "residual", F32, 2)
     _dev(weight, "weight", (F32, BF16), 1)
-    _check_split(pending, "pending", residual.shape)
+    if pending is not None:
+        _check_split(pending, "pending", residual.shape)
     if stream is not None:
         _dev(stream, "stream", F32, 2)
         if stream.shape != residual.shape:
             raise ValueError("the stream must have the residual's shape")
+    if next_out is not None:
+        _dev(next_out, "next_out", BF16, 2)
+        if next_out.shape != residual.shape:
+            raise ValueError("next_out must have the residual's shape")
     if weight.shape[0] != residual.shape[1]:
         raise ValueError("the weight must have the residual's width")
-    _check(library().ms_normed_add_pending(residual.data_ptr(), _ptr(stream), pending.parts.data_ptr(), pending.splits, pending.stride,
+    _check(library().ms_normed_add_pending(residual.data_ptr(), _ptr(stream), pending.parts.data_ptr() if pending is not None else None,
+                                           pending.splits if pending is not None else 0, pending.stride if pending is not None else 0,
                                            weight.data_ptr(), int(weight.dtype == BF16), residual.shape[0], residual.shape[1], float(eps),
-                                           _stream()), "normed_add_pending")
+                                           _ptr(next_out), int(clear), _stream()), "normed_add_pending")
 
 
 def scale_(x: torch.Tensor, factor: float) -> torch.Tensor:

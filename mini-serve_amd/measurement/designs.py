@@ -146,8 +146,8 @@ def measure(config: dict, dtype: str, prefill_tokens: int, batch: int, context: 
     out = {"prefill_tok_s": round(prefill_tokens / prefill_s, 1), "prefill_ms": round(prefill_s * 1e3, 3),
            "prefill_tflops": round(model.step_flops([(prefill_tokens, 0)]) / prefill_s / 1e12, 1),
            "decode_tok_s": round(batch / decode_s, 1), "decode_ms_per_step": round(decode_s * 1e3, 4),
-           "decode_weight_gbs": round(model.decode_read_bytes() / decode_s / 1e9, 1),
-           "weights_gb": round(model.decode_read_bytes() / 1e9, 3)}
+           "decode_weight_gbs": round(model.decode_read_bytes(batch) / decode_s / 1e9, 1),
+           "weights_gb": round(model.decode_read_bytes(batch) / 1e9, 3)}
     del runner, model
     torch.cuda.empty_cache()
     return out

@@ -176,6 +176,11 @@ class Part:
         """Bytes of weights a decode step reads from this part (for the bandwidth model)."""
         return 0
 
+    def step_read_bytes(self, tokens: int) -> int:
+        """Bytes of weights a step of ``tokens`` single tokens reads from this part: ``parameters_bytes()`` unless what
+        is read depends on the tokens (a part that routes them to some of its weights)."""
+        return self.parameters_bytes()
+
     def flops(self, rows) -> int:
         """Floating-point operations of one pass over ``rows``: a list of ``(new tokens, tokens already in
         the cache)`` per request; a multiply-add counts two. What a measurement divides by its time."""
@@ -188,10 +193,11 @@ class Norm(Part):
         also brought up to date in place; with ``rows`` the stream is not read again and stays as it is."""
         raise NotImplementedError
 
-    def add_normed(self, residual, stream, pending=None) -> None:
+    def add_normed(self, residual, stream, pending=None, next_out=None, clear=False) -> None:
         """``residual += norm(stream + pending)`` row by row, both float32 and of one shape (``pending``: a sum the
         sublayer left to be added to its stream): the norm of a layer that norms what a sublayer puts out instead of
-        what it reads."""
+        what it reads. ``next_out`` (the compute dtype, same shape; None: not wanted) receives the new residual, and
+        with ``clear`` the stream is zero afterwards."""
         raise NotImplementedError(f"norm {self.kind!r} cannot norm a sublayer's output into the residual stream")
 
 

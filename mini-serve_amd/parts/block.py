@@ -73,8 +73,8 @@ class ParallelBlock(Block):
 @register("block", "outnorm")
 class OutputNormBlock(Block):
     """``h += norm1(mixer(h)); h += norm2(feed_forward(h))``: the sublayers read the stream itself, and what they put
-    out is normed before it joins the stream. Each sublayer adds into a stream of its own that starts at zero; the
-    norm's ``add_normed`` folds it into the residual stream. A layer without a feed-forward has no second norm
+    out is normed before it joins the stream. Each sublayer adds into a stream that starts at zero; the norm's
+    ``add_normed`` folds it into the residual stream and leaves it zero for the next sublayer. A layer without a feed-forward has no second norm
     (``ffn_norm`` None); ``spare`` then names norm tensors ``{name: width}`` that a checkpoint may still carry for it.
     ``mixer_scale`` / ``ffn_scale`` (optional) name a tensor ``[width]`` each by which the normed output is multiplied
     element by element before it joins the stream (a layer scale): ``h += scale * norm(sublayer(h))``. It is folded into
@@ -109,17 +109,25 @@ class OutputNormBlock(Block):
             if self.spec.get("ffn_scale"):
                 self.ffn_norm.fold_scale(tensors[self.spec["ffn_scale"]])
 
-    def _sublayer(self, run, norm, residual) -> None:
-        ops = self.rt.ops
-        own = torch.zeros_like(residual)
-        pending = run(ops.cast(residual, self.rt.dtype), own)
-        norm.add_normed(residual, own, pending)  # the sublayer's output is its stream plus what it left pending
-
     def forward(self, residual, batch, cache, state, pending=None):
-        self.rt.ops.add_pending(residual, pending)
-        self._sublayer(lambda x, own: self.mixer.forward(x, batch, cache, state, own), self.mixer_norm, residual)
-        if self.ffn_norm is not None:
-            self._sublayer(lambda x, own: self.feed_forward.forward(x, own), self.ffn_norm, residual)
+        ops, dtype = self.rt.ops, self.rt.dtype
+        ops.add_pending(residual, pending)
+        # The stream the sublayers add into is zeroed once per pass: the norm's kernel leaves it zero again. The same
+        # kernel hands the feed-forward the new residual in the compute dtype, so that it needs no cast of its own.
+        key = ("outnorm_stream", tuple(residual.shape))
+        own = batch.memo.get(key)
+        if own is None:
+            own = batch.memo[key] = torch.zeros_like(residual)
+        x = ops.cast(residual, dtype)
+        first = self.mixer.forward(x, batch, cache, state, own)
+        if self.ffn_norm is None:
+            self.mixer_norm.add_normed(residual, own, first, clear=True)
+            return None
+        rounded = dtype == torch.bfloat16
+        x = torch.empty_like(x) if rounded else residual
+        self.mixer_norm.add_normed(residual, own, first, next_out=x if rounded else None, clear=True)
+        second = self.feed_forward.forward(x, own)
+        self.ffn_norm.add_normed(residual, own, second, clear=True)
         return None
 
     def parameters_bytes(self) -> int:

@@ -199,6 +199,14 @@ class MixtureMLP(FeedForward):
         own = self.router.numel() * self.router.element_size() + self.top * per_expert
         return own + (self.shared.parameters_bytes() if self.shared is not None else 0)
 
+    def step_read_bytes(self, tokens: int) -> int:
+        """The router, the shared expert and the experts that ``tokens`` tokens are expected to choose between them when
+        every choice of ``top`` is as likely as any other: ``E (1 - (1 - top / E) ** tokens)`` experts."""
+        per_expert = sum(t[0].numel() * t.element_size() for t in (self.gate, self.up, self.down))
+        distinct = self.num_experts * (1.0 - (1.0 - self.top / self.num_experts) ** max(1, tokens))
+        own = self.router.numel() * self.router.element_size() + int(round(distinct * per_expert))
+        return own + (self.shared.parameters_bytes() if self.shared is not None else 0)
+
     def flops(self, rows) -> int:
         tokens = sum(n for n, _ in rows)
         own = 2 * tokens * self.hidden * self.num_experts + 2 * tokens * self.top * 3 * self.hidden * self.inter

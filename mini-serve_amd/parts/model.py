@@ -158,11 +158,12 @@ class DecoderModel:
             total += b.flops(rows) + b.mixer.flops(rows) + b.feed_forward.flops(rows)
         return total
 
-    def decode_read_bytes(self) -> int:
-        """Bytes of weights one decode step reads: every run-order entry's layer once, the final
-        norm and the head (embedding rows are only gathered)."""
+    def decode_read_bytes(self, tokens: int = 1) -> int:
+        """Bytes of weights one decode step of ``tokens`` requests reads: every run-order entry's layer once, the final
+        norm and the head (embedding rows are only gathered). Only parts that route tokens to some of their weights read
+        more for more tokens."""
         total = self.final_norm.parameters_bytes() + self.head.parameters_bytes()
         for e in self.spec.run_order:
             b = self.blocks[e.layer]
-            total += b.parameters_bytes() + b.mixer.parameters_bytes() + b.feed_forward.parameters_bytes()
+            total += b.parameters_bytes() + b.mixer.step_read_bytes(tokens) + b.feed_forward.step_read_bytes(tokens)
         return total

@@ -46,8 +46,10 @@ class RMSNorm(Norm):
         Returns the compute dtype, ``[T or len(rows), width]``."""
         return self.rt.ops.rmsnorm(x, self.weight, self.eps, self.rt.dtype, rows, add)
 
-    def add_normed(self, residual, stream, pending=None) -> None:
-        self.rt.ops.normed_add(residual, stream, self.weight, self.eps, pending)
+    def add_normed(self, residual, stream, pending=None, next_out=None, clear=False) -> None:
+        """``residual += norm(stream + pending)``; ``next_out`` (bfloat16) receives the new residual rounded, and with
+        ``clear`` the stream is left zero (both inside the norm's kernel)."""
+        self.rt.ops.normed_add(residual, stream, self.weight, self.eps, pending, next_out, clear)
 
     def parameters_bytes(self) -> int:
         return self.weight.numel() * self.weight.element_size()
