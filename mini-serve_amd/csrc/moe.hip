@@ -8,7 +8,9 @@
 //
 // A pair's result depends on its own row and its expert's weights alone (every output element is one dot product, summed
 // in an order that its place in a tile does not change), so neither the order of the pairs inside an expert's run nor
-// what else the step holds changes a token's result; the sum over a token's choices runs in the order of the choices.
+// which other pairs the step holds changes a token's result; how many pairs it holds picks the size of the tiles, and
+// the kernels of different tile sizes add in different orders (rounding of float32 sums). The sum over a token's choices
+// runs in the order of the choices.
 #include "common.h"
 
 #define MOE_MAX_EXPERTS 512
@@ -16,10 +18,12 @@
 
 // ---------------------------------------------------------------------------------------------
 // Routing: z = logits[t] + bias; the `top` largest z (ties: the lower index), largest first; weights = softmax over
-// those alone. One wave per token.
+// those alone. One wave per token. The logits may come as `splits` partial sums `stride` floats apart (the router's
+// product over few rows leaves them so), added here in ascending order.
 template <typename TB>
-__global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits, int ld, const TB* __restrict__ bias,
-                                                        int T, int E, int top, int* __restrict__ ids, float* __restrict__ weights) {
+__global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits, int ld, int splits, size_t stride,
+                                                        const TB* __restrict__ bias, int T, int E, int top,
+                                                        int* __restrict__ ids, float* __restrict__ weights) {
   const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
   const int t = blockIdx.x * 4 + wave;
   if (t >= T) return;
@@ -27,7 +31,7 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
 #pragma unroll
   for (int i = 0; i < MOE_MAX_EXPERTS / WAVE; ++i) {
     const int e = lane + i * WAVE;
-    z[i] = e < E ? logits[(size_t)t * ld + e] + (bias ? to_f32(bias[e]) : 0.f) : -INFINITY;
+    z[i] = e < E ? sum_splits(logits + (size_t)t * ld + e, splits, stride) + (bias ? to_f32(bias[e]) : 0.f) : -INFINITY;
   }
   float chosen = 0.f;  // lane j keeps the j-th chosen logit
   for (int j = 0; j < top; ++j) {
@@ -56,14 +60,16 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
   if (lane < top) weights[(size_t)t * top + lane] = expf(chosen - m) / sum;
 }
 
-extern "C" int ms_moe_route(const float* logits, int ld, const void* bias, int bias_is_bf16, int T, int E, int top, int* ids,
-                            float* weights, hipStream_t st) {
+extern "C" int ms_moe_route(const float* logits, int ld, int splits, long long stride, const void* bias, int bias_is_bf16, int T,
+                            int E, int top, int* ids, float* weights, hipStream_t st) {
   if (T <= 0) return MS_OK;
-  if (logits == nullptr || ids == nullptr || weights == nullptr || E < 1 || top < 1 || top > E || ld < E) return MS_BAD_ARG;
+  if (logits == nullptr || ids == nullptr || weights == nullptr || E < 1 || top < 1 || top > E || ld < E || splits < 1 ||
+      (splits > 1 && stride < (long long)T * ld))
+    return MS_BAD_ARG;
   if (E > MOE_MAX_EXPERTS || top > MOE_MAX_TOP) return MS_UNSUPPORTED;
   const unsigned blocks = (unsigned)((T + 3) / 4);
-  if (bias_is_bf16) moe_route_kernel<bf16><<<blocks, 256, 0, st>>>(logits, ld, (const bf16*)bias, T, E, top, ids, weights);
-  else moe_route_kernel<float><<<blocks, 256, 0, st>>>(logits, ld, (const float*)bias, T, E, top, ids, weights);
+  if (bias_is_bf16) moe_route_kernel<bf16><<<blocks, 256, 0, st>>>(logits, ld, splits, (size_t)stride, (const bf16*)bias, T, E, top, ids, weights);
+  else moe_route_kernel<float><<<blocks, 256, 0, st>>>(logits, ld, splits, (size_t)stride, (const float*)bias, T, E, top, ids, weights);
   return launch_status();
 }
 
@@ -181,21 +187,29 @@ __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(
   moe_floatx4 acc1[NT], acc2[NT];
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) acc1[nt] = acc2[nt] = moe_floatx4{0.f, 0.f, 0.f, 0.f};
+  // 64 k a step: a lane takes 16 consecutive k of its rows (two loads of 16 bytes: a wave reads a whole 128-byte line
+  // of every row) and multiplies them in two products. Both operands are cut the same way, so the sum is over
+  // every k once; within a step the order of k is that of the lanes' runs.
 #pragma unroll(4 / NT)
-  for (int k0 = 0; k0 < K; k0 += 32) {
-    const int kk = k0 + grp * 8;  // the lane's eight elements of this step
-    const moe_bf16x8 av = moe_load<ALIGNED>(ap, kk, K, row_ok);
-    moe_bf16x8 b1[NT], b2[NT];
+  for (int k0 = 0; k0 < K; k0 += 64) {
+    const int kk = k0 + grp * 16;  // the lane's sixteen elements of this step
+    moe_bf16x8 av[2], b1[NT][2], b2[NT][2];
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-      b1[nt] = moe_load<ALIGNED>(wp1[nt], kk, K, col_ok[nt]);
-      if (GATED) b2[nt] = moe_load<ALIGNED>(wp2[nt], kk, K, col_ok[nt]);
+    for (int u = 0; u < 2; ++u) {
+      av[u] = moe_load<ALIGNED>(ap, kk + 8 * u, K, row_ok);
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+        b1[nt][u] = moe_load<ALIGNED>(wp1[nt], kk + 8 * u, K, col_ok[nt]);
+        if (GATED) b2[nt][u] = moe_load<ALIGNED>(wp2[nt], kk + 8 * u, K, col_ok[nt]);
+      }
     }
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-      acc1[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, b1[nt], acc1[nt], 0, 0, 0);
-      if (GATED) acc2[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, b2[nt], acc2[nt], 0, 0, 0);
-    }
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+        acc1[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[u], b1[nt][u], acc1[nt], 0, 0, 0);
+        if (GATED) acc2[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[u], b2[nt][u], acc2[nt], 0, 0, 0);
+      }
   }
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
@@ -226,7 +240,7 @@ __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(
 //   GATED: the tile's weight rows are blocks of 16 gate rows and 16 up rows in turn (64 columns of h a block), so that a
 //          lane's fragments 2 i and 2 i + 1 are gate and up of the same four outputs.
 // Pairs past the tile's count read the tile's last pair, weight rows past N the last row: their results are not stored.
-// Every output element is the same chain of products over k as in the kernel above, whatever the tile.
+// Every output element is one chain of products over k in ascending slabs, whatever the tile and the pair's place in it.
 template <int N_> __device__ __forceinline__ void moe_wait_loads() {
   __builtin_amdgcn_s_waitcnt((N_ & 15) | ((N_ >> 4) << 14) | (7 << 4) | (15 << 8));  // vmcnt alone
 }

@@ -99,7 +99,7 @@ _SIGNATURES = {
     "ms_head_prepare_store": [_c_void, _c_int, _c_void, _c_int, _c_void, _c_void, _c_void, _c_int, _c_int, _c_float, _c_void, _c_int,
                               _c_int, _c_void, _c_int, _c_float, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
                               _c_void],
-    "ms_moe_route": [_c_void, _c_int, _c_void, _c_int, _c_int, _c_int, _c_int, _c_void, _c_void, _c_void],
+    "ms_moe_route": [_c_void, _c_int, _c_int, _c_ll, _c_void, _c_int, _c_int, _c_int, _c_int, _c_void, _c_void, _c_void],
     "ms_moe_plan": [_c_void, _c_int, _c_int, _c_int, _c_int, _c_void, _c_void, _c_void, _c_void, _c_void],
     "ms_moe_gemm": [_c_void, _c_int, _c_void, _c_void, _c_void, _c_int, _c_int, _c_void, _c_void, _c_void, _c_void, _c_void,
                     _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
@@ -470,12 +470,18 @@ MOE_SMALL_TILE_PAIRS = 16  # (token, expert) pairs per expert, on average, up to
 MOE_LARGE_TILE_PAIRS = 128  # ... and from which it runs 128-pair tiles (widths that are multiples of 64)
 
 
-def moe_route(logits: torch.Tensor, bias: torch.Tensor | None, top: int):
+def moe_route(logits, bias: torch.Tensor | None, top: int):
     """Per row of the float32 router logits ``[T, E]`` (plus ``bias [E]``): the ``top`` experts with the largest values,
     largest first (ties: the lower index), as int32 ``[T, top]``, and the softmax over those values alone, float32
-    ``[T, top]``."""
-    _dev(logits, "logits", F32, 2)
-    t, e = logits.shape
+    ``[T, top]``. The logits may be a ``SplitSum``: the kernel adds the partial sums itself."""
+    if isinstance(logits, SplitSum):
+        parts, splits, stride = logits.parts, logits.splits, logits.stride
+        _dev(parts, "logits", F32, 3)
+        t, e = logits.shape
+    else:
+        _dev(logits, "logits", F32, 2)
+        parts, splits, stride = logits, 1, 0
+        t, e = logits.shape
     if not 1 <= top <= e:
         raise ValueError(f"top {top} of {e} experts")
     if e > MOE_MAX_EXPERTS or top > MOE_MAX_TOP:
@@ -484,10 +490,10 @@ def moe_route(logits: torch.Tensor, bias: torch.Tensor | None, top: int):
         _dev(bias, "bias", (F32, BF16), 1)
         if bias.shape[0] != e:
             raise ValueError(f"the router's bias has {bias.shape[0]} elements for {e} experts")
-    ids = torch.empty((t, top), dtype=I32, device=logits.device)
-    weights = torch.empty((t, top), dtype=F32, device=logits.device)
-    _check(library().ms_moe_route(logits.data_ptr(), e, _ptr(bias), int(bias is not None and bias.dtype == BF16), t, e, top,
-                                  ids.data_ptr(), weights.data_ptr(), _stream()), "moe_route")
+    ids = torch.empty((t, top), dtype=I32, device=parts.device)
+    weights = torch.empty((t, top), dtype=F32, device=parts.device)
+    _check(library().ms_moe_route(parts.data_ptr(), e, splits, stride, _ptr(bias), int(bias is not None and bias.dtype == BF16), t, e,
+                                  top, ids.data_ptr(), weights.data_ptr(), _stream()), "moe_route")
     return ids, weights
 
 

@@ -186,7 +186,7 @@ class MixtureMLP(FeedForward):
     def forward(self, x, residual):
         ops = self.rt.ops
         pending = self.shared.forward(x, residual) if self.shared is not None else None
-        logits = ops.linear(x, self.router, out_dtype=torch.float32)
+        logits = ops.linear(x, self.router, out_dtype=torch.float32, defer=True)  # few rows: partial sums, added by the routing
         ids, weights = ops.moe_route(logits, self.bias, self.top)
         xe = ops.cast(x, self.gate.dtype)  # experts stored in 32-bit compute in 32-bit
         ops.moe_experts(xe, ids, weights, self.gate, self.up, self.down, self.activation, residual)

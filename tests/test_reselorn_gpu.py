@@ -298,6 +298,14 @@ def test_routing(experts, top):
     if experts > 2:  # with no bias row 6 is all ties: the first `top` experts in order, equal weights
         ids, wts = o.moe_route(dev(z), None, top)
         assert ids[6].tolist() == list(range(top)) and np.allclose(wts[6].cpu().numpy(), 1.0 / top)
+    # logits that arrive as partial sums of the router's product: the kernel adds them in ascending order
+    parts = rng.normal(size=(11, T, experts)).astype(np.float32)
+    total = np.zeros((T, experts), np.float32)
+    for part in parts:
+        total = total + part
+    ids, wts = o.moe_route(o.SplitSum(dev(parts)), None, top)
+    want_ids, want_wts = o.moe_route(dev(total), None, top)
+    assert torch.equal(ids, want_ids) and torch.equal(wts, want_wts)
     with pytest.raises(ValueError):
         o.moe_route(dev(z), None, experts + 1)
 
