@@ -325,12 +325,15 @@ __global__ __launch_bounds__(256, 2) void moe_gemm_bf16_lds_kernel(
       for (int j = 0; j < FM; ++j) xf[t][j] = *reinterpret_cast<const moe_bf16x8*>(stage + x_off + j * 16 * ROW_BYTES + slot);
     }
     __builtin_amdgcn_sched_barrier(0);
+    // an expert's last tile is seldom full: runs of 16 pairs past its count are not multiplied (the same for a whole wave)
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
-      for (int i = 0; i < FN; ++i)
+      for (int j = 0; j < FM; ++j) {
+        if (wm + j * 16 >= count) continue;
 #pragma unroll
-        for (int j = 0; j < FM; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[t][i], xf[t][j], acc[i][j], 0, 0, 0);
+        for (int i = 0; i < FN; ++i) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[t][i], xf[t][j], acc[i][j], 0, 0, 0);
+      }
   }
 
   const bool vec = N % 4 == 0;
