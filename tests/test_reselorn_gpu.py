@@ -346,6 +346,30 @@ def test_experts(width, ff, experts, top, dtype):
         close(stream, want, dtype, f"{T} tokens", tol=3e-5 if dtype == torch.float32 else 6e-3)
 
 
+@pytest.mark.parametrize("width", [7, 1000, 2048, 9000])
+def test_output_norm_with_a_rounded_copy_and_a_cleared_stream(width):
+    """``residual += y / rms(y) * w`` where ``y`` is a stream, partial sums, or both; the kernel may also hand back the new
+    residual in bfloat16 and leave the stream zero. Widths below, at and beyond what a thread keeps in registers."""
+    o = ops()
+    rng = np.random.default_rng(width)
+    rows = 5
+    r, y, w = rng.normal(size=(rows, width)), rng.normal(size=(rows, width)) * 4, rng.normal(size=width) + 1
+    parts = rng.normal(size=(13, rows, width))
+    for stream, pending in ((y, None), (y, parts), (None, parts)):
+        total = (0 if stream is None else y) + (0 if pending is None else parts.sum(0))
+        want = r + total / np.sqrt((total ** 2).mean(-1, keepdims=True) + 1e-5) * w
+        for copy, clear in ((False, False), (True, True), (False, True), (True, False)):
+            res = dev(r)
+            st = None if stream is None else dev(stream)
+            nxt = torch.full((rows, width), 7.0, dtype=torch.bfloat16, device=DEV) if copy else None
+            o.normed_add(res, st, dev(w), 1e-5, None if pending is None else o.SplitSum(dev(parts)), nxt, clear)
+            close(res, want, torch.float32, tol=3e-5)
+            if copy:
+                assert torch.equal(nxt, res.to(torch.bfloat16)), "the copy is the new residual, rounded once"
+            if st is not None:
+                assert (not clear and torch.equal(st, dev(stream))) or (clear and not st.any()), "the stream afterwards"
+
+
 # ---------------------------------------------------------------- whole models
 
 
