@@ -2,8 +2,8 @@
 key/value heads (grouped, one group, none shared), query/key sizes unlike value sizes, sizes that are no multiple of 8,
 heads wider than 256, a rotation over the whole head, over a part of it and none, slowed and plain frequencies, windows
 shorter and longer than a page and none at all, blended values that start at the first layer or later, layers that
-do not blend, dense layers, mixtures with and without a shared expert, one expert, every expert chosen, one chosen, and
-layers without a feed-forward.
+do not blend, dense layers, mixtures with and without a shared expert, one expert, every expert chosen, one chosen,
+layers without a feed-forward, and windows of one token, of two and of exactly a page.
 
 ``make_folder`` draws random weights and then makes them telling: sinks and blend weights large enough to matter, and a
 router whose choice is exact in every number format (it reads only the stream's last channels, which the layer scales
@@ -79,6 +79,13 @@ RESELORN = {
         attention(4, 2, 96, 32, 0.1, {"base": 1000.0, "dims": 32}, size=40, v_mix=True, mlp=moe(9, 3, 32, None)),
         attention(2, 2, 128, 32, 0.09, slowed(1000.0, 64, 2.0, 48, 4.0, 0.5), size=50, v_mix=True, mlp=dense(64)),
     ]), 34, Init(0.1, (0.6, 1.4))),
+    # values that are one: a window of a single token and of two, one rotated pair, one chosen expert of two, every one of
+    # three, one head, a factor that slows nothing, a window of exactly a page
+    "rsE": (model(53, 40, 1e-4, [
+        attention(2, 1, 8, 8, 1.0, {"base": 50.0, "dims": 2}, size=1, v_mix=True, mlp=moe(2, 1, 8, 8)),
+        attention(2, 2, 8, 8, 0.7, slowed(50.0, 8, 1.0, 8, 1.0, 1.0), size=2, v_mix=False, mlp=moe(3, 3, 8)),
+        attention(1, 1, 16, 8, 0.5, None, size=16, v_mix=True, mlp=dense(8)),
+    ]), 35, Init(0.15, (0.6, 1.4))),
 }
 
 

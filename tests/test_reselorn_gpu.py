@@ -184,7 +184,8 @@ CUTS = ([400], [150] + [1] * 250, [2, 3, 64, 5, 2, 31, 1, 1, 190, 1, 100])
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("hq,hk,d,e,size,dims", [(4, 2, 32, 24, 37, 16), (3, 1, 10, 6, 16, 6), (8, 2, 96, 32, 100, 32), (6, 3, 64, 64, 0, 64),
-                                                 (2, 2, 272, 16, 80, 272), (16, 1, 128, 128, 70, 64), (4, 4, 40, 72, 17, 0)])
+                                                 (2, 2, 272, 16, 80, 272), (16, 1, 128, 128, 70, 64), (4, 4, 40, 72, 17, 0),
+                                                 (4, 2, 32, 24, 1, 16), (2, 1, 64, 64, 2, 32), (4, 2, 128, 128, 16, 64)])
 def test_grouped_attention_behind_the_preparation(hq, hk, d, e, size, dims, dtype):
     """Projection rows through rotation, norm, blend and store into pages, then attention with sinks inside a window, in
     cuts of every kind. Queries and keys have unit length here, so a key stands out by its direction: for the last query
@@ -221,8 +222,9 @@ def test_grouped_attention_behind_the_preparation(hq, hk, d, e, size, dims, dtyp
     if size:  # the outer key would take most of the weight if it were seen
         seen = plain_attention(qr, kr, vr, scale, size + 1, sinks)
         assert np.abs(seen - want)[T - 1].max() > 0.2 * np.abs(want[T - 1]).max()
-        lost = plain_attention(qr, kr, vr, scale, size - 1, sinks)
-        assert np.abs(lost - want)[T - 1].max() > 0.05 * np.abs(want[T - 1]).max()
+        if size > 1:  # (a window of one token sees itself alone: nothing narrower exists)
+            lost = plain_attention(qr, kr, vr, scale, size - 1, sinks)
+            assert np.abs(lost - want)[T - 1].max() > 0.05 * np.abs(want[T - 1]).max()
     pages = [int(p) for p in rng.permutation(30)[: -(-T // PAGE)]]
     kc = torch.zeros((31, hk, PAGE, d), dtype=dtype, device=DEV)
     vc = torch.zeros((31, hk, e, PAGE), dtype=dtype, device=DEV)
@@ -499,7 +501,7 @@ def test_a_router_that_reads_the_whole_stream(tmp_path, folders):
     check_logits(got, R.forward(cfg, w, toks), "float32", "a router over the whole stream")
 
 
-@pytest.mark.parametrize("name", sorted(RESELORN))
+@pytest.mark.parametrize("name", sorted(set(RESELORN) - {"rsE"}))  # (rsE's ones leave some options without effect, on purpose)
 def test_the_models_show_what_is_left_out(name, folders, plain_logits):
     """What the comparisons are worth: with these weights a window one token off, a sink left out, values that are not
     blended, plain frequencies for slowed ones, a router without its bias, one choice fewer, a missing shared expert or a missing layer scale moves the logits by far more than the
@@ -530,7 +532,7 @@ def test_the_models_show_what_is_left_out(name, folders, plain_logits):
         if m["v_mix"] and blending:
             assert moved(weights=without(f"l{i}.mix.vmix")) > floor, (name, i, "blend")
         blending = blending or m["v_mix"]
-        if m.get("rot") and m["rot"].get("scaling"):
+        if m.get("rot") and m["rot"].get("scaling") and m["rot"]["scaling"]["factor"] != 1.0:  # (a factor of one slows nothing)
             sc = mo["rot"].pop("scaling")
             assert moved(off) > floor, (name, i, "slowed frequencies")
             mo["rot"]["scaling"] = sc
