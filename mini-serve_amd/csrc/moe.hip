@@ -158,7 +158,7 @@ template <bool ALIGNED> __device__ __forceinline__ moe_bf16x8 moe_load(const bf1
   return x.v;
 }
 
-template <bool GATED, bool ALIGNED, int NT>
+template <bool GATED, bool ALIGNED, int NT, bool KSPLIT = false>
 __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(
     const bf16* __restrict__ a, int lda, const bf16* __restrict__ w1, const bf16* __restrict__ w2, void* __restrict__ out,
     const int* __restrict__ order, const int* __restrict__ tile_expert, const int* __restrict__ tile_start,
@@ -168,8 +168,13 @@ __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(
   const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE, l16 = lane % 16, grp = lane / 16;
   const bool by_rows = tile_rows == 64;
   const int m0 = by_rows ? wave * 16 : 0;
-  const int n0 = by_rows ? blockIdx.y * (16 * NT) : (blockIdx.y * 4 + wave) * (16 * NT);
+  // KSPLIT (16-pair tiles): the block's four waves share its 16 NT columns and take a quarter of K each (a multiple of 64),
+  // so that four times the waves stream a step's weights; their sums meet in LDS and are added in wave order.
+  const int n0 = (by_rows || KSPLIT) ? blockIdx.y * (16 * NT) : (blockIdx.y * 4 + wave) * (16 * NT);
   if (m0 >= count || n0 >= N) return;
+  const int k_quarter = ((K + 3) / 4 + 63) / 64 * 64;
+  const int k_lo = KSPLIT ? min(K, wave * k_quarter) : 0;
+  const int k_hi = KSPLIT ? min(K, k_lo + k_quarter) : K;
   const int e = tile_expert[blockIdx.x], start = tile_start[blockIdx.x];
   const bool row_ok = m0 + l16 < count;
   const int place = start + m0 + (row_ok ? l16 : 0);
@@ -191,16 +196,16 @@ __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(
   // of every row) and multiplies them in two products. Both operands are cut the same way, so the sum is over
   // every k once; within a step the order of k is that of the lanes' runs.
 #pragma unroll(4 / NT)
-  for (int k0 = 0; k0 < K; k0 += 64) {
+  for (int k0 = k_lo; k0 < k_hi; k0 += 64) {
     const int kk = k0 + grp * 16;  // the lane's sixteen elements of this step
     moe_bf16x8 av[2], b1[NT][2], b2[NT][2];
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
-      av[u] = moe_load<ALIGNED>(ap, kk + 8 * u, K, row_ok);
+      av[u] = moe_load<ALIGNED>(ap, kk + 8 * u, k_hi, row_ok);
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt) {
-        b1[nt][u] = moe_load<ALIGNED>(wp1[nt], kk + 8 * u, K, col_ok[nt]);
-        if (GATED) b2[nt][u] = moe_load<ALIGNED>(wp2[nt], kk + 8 * u, K, col_ok[nt]);
+        b1[nt][u] = moe_load<ALIGNED>(wp1[nt], kk + 8 * u, k_hi, col_ok[nt]);
+        if (GATED) b2[nt][u] = moe_load<ALIGNED>(wp2[nt], kk + 8 * u, k_hi, col_ok[nt]);
       }
     }
 #pragma unroll
@@ -210,6 +215,29 @@ __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(
         acc1[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[u], b1[nt][u], acc1[nt], 0, 0, 0);
         if (GATED) acc2[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[u], b2[nt][u], acc2[nt], 0, 0, 0);
       }
+  }
+  if constexpr (KSPLIT) {
+    __shared__ float meet[3][GATED ? 2 * NT : NT][4][WAVE];
+    if (wave > 0) {
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          meet[wave - 1][nt][r][lane] = acc1[nt][r];
+          if (GATED) meet[wave - 1][NT + nt][r][lane] = acc2[nt][r];
+        }
+    }
+    __syncthreads();
+    if (wave > 0) return;
+#pragma unroll
+    for (int w = 0; w < 3; ++w)
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          acc1[nt][r] += meet[w][nt][r][lane];
+          if (GATED) acc2[nt][r] += meet[w][NT + nt][r][lane];
+        }
   }
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
@@ -498,10 +526,17 @@ extern "C" int ms_moe_gemm(const void* a, int lda, const void* w1, const void* w
       const long busy = max_tiles / 2 + 1;  // about half of the launched tiles hold pairs
       while (nt > 1 && busy * ((N + 64 * nt - 1) / (64 * nt)) < 1024) nt /= 2;
     }
+    const bool aligned = K % 8 == 0 && lda % 8 == 0 && (size_t)a % 16 == 0 && (size_t)w1 % 16 == 0 && (!gated || (size_t)w2 % 16 == 0);
+    // still few blocks at the narrowest columns: the waves of a block share 16 columns and split K
+    if (tile_rows == 16 && nt == 1 && aligned && K >= 512 && (max_tiles / 2 + 1) * ((N + 63) / 64) < 2048 && (N + 15) / 16 <= 65535) {
+      const dim3 grid(max_tiles, (N + 15) / 16);
+      if (gated) moe_gemm_bf16_kernel<true, true, 1, true><<<grid, 256, 0, st>>>((const bf16*)a, lda, (const bf16*)w1, (const bf16*)w2, out, order, tile_expert, tile_start, tile_count, pair_weight, top, N, K, tile_rows, act);
+      else moe_gemm_bf16_kernel<false, true, 1, true><<<grid, 256, 0, st>>>((const bf16*)a, lda, (const bf16*)w1, (const bf16*)w2, out, order, tile_expert, tile_start, tile_count, pair_weight, top, N, K, tile_rows, act);
+      return launch_status();
+    }
     const int cols = tile_rows == 64 ? 64 : 64 * nt;
     const dim3 grid(max_tiles, (N + cols - 1) / cols);
     if (grid.y > 65535) return MS_BAD_ARG;
-    const bool aligned = K % 8 == 0 && lda % 8 == 0 && (size_t)a % 16 == 0 && (size_t)w1 % 16 == 0 && (!gated || (size_t)w2 % 16 == 0);
 #define MOE(G, A, T) moe_gemm_bf16_kernel<G, A, T><<<grid, 256, 0, st>>>((const bf16*)a, lda, (const bf16*)w1, (const bf16*)w2, out, order, tile_expert, tile_start, tile_count, pair_weight, top, N, K, tile_rows, act)
 #define MOE_NT(G, A) do { if (nt == 4) MOE(G, A, 4); else if (nt == 2) MOE(G, A, 2); else MOE(G, A, 1); } while (0)
     if (gated) { if (aligned) MOE_NT(true, true); else MOE_NT(true, false); }

@@ -314,11 +314,12 @@ def test_routing(experts, top):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("width,ff,experts,top", [(24, 10, 3, 3), (90, 50, 7, 2), (64, 32, 1, 1), (128, 64, 20, 4), (136, 72, 40, 1), (96, 264, 5, 5),
-                                                  (128, 192, 4, 2), (192, 64, 3, 1)])
+                                                  (128, 192, 4, 2), (192, 64, 3, 1), (512, 520, 6, 2)])
 def test_experts(width, ff, experts, top, dtype):
     """The sorted products against a loop over tokens and choices, for steps of one token to several tiles per expert, with
     choices that leave experts idle and choices that send every token to one. Widths that are multiples of 64 run the tiles
-    staged through LDS (64 and 128 pairs), with output widths that end inside a tile's columns."""
+    staged through LDS (64 and 128 pairs), with output widths that end inside a tile's columns; widths from 512 on split K
+    over a block's waves where the step has few tokens."""
     o = ops()
     rng = np.random.default_rng(width + experts)
     gate, up, down = rng.normal(size=(experts, ff, width)), rng.normal(size=(experts, ff, width)), rng.normal(size=(experts, width, ff))
