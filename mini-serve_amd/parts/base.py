@@ -187,6 +187,12 @@ class Part:
         return 0
 
 
+# ``batch.memo`` key under which a block may leave the residual stream as it stands after the block, in the compute dtype,
+# for the block that runs next (which would otherwise cast it). The model drops what the block that just ran did not
+# leave itself, so an entry is never older than one block.
+ROUNDED_RESIDUAL = "residual_in_compute_dtype"
+
+
 class Norm(Part):
     def forward(self, x, rows=None, add=None):
         """Normalise rows of the float32 ``x`` plus ``add`` (a pending sum). Without ``rows``, ``x`` is

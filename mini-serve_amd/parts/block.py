@@ -7,7 +7,7 @@ from __future__ import annotations
 import torch
 
 from ..config.spec import PartSpec
-from .base import Block, TensorSpec
+from .base import ROUNDED_RESIDUAL, Block, TensorSpec
 from .registry import part_class, register
 
 
@@ -113,21 +113,25 @@ class OutputNormBlock(Block):
         ops, dtype = self.rt.ops, self.rt.dtype
         ops.add_pending(residual, pending)
         # The stream the sublayers add into is zeroed once per pass: the norm's kernel leaves it zero again. The same
-        # kernel hands the feed-forward the new residual in the compute dtype, so that it needs no cast of its own.
+        # kernel hands the next reader (the feed-forward, the next block) the new residual in the compute dtype, so that
+        # a layer casts the stream only where the block before it left no such copy.
         key = ("outnorm_stream", tuple(residual.shape))
         own = batch.memo.get(key)
         if own is None:
             own = batch.memo[key] = torch.zeros_like(residual)
-        x = ops.cast(residual, dtype)
-        first = self.mixer.forward(x, batch, cache, state, own)
-        if self.ffn_norm is None:
-            self.mixer_norm.add_normed(residual, own, first, clear=True)
-            return None
         rounded = dtype == torch.bfloat16
+        x = batch.memo.pop(ROUNDED_RESIDUAL, None)
+        if pending is not None or x is None or x.shape != residual.shape or x.dtype != dtype:
+            x = ops.cast(residual, dtype)
+        first = self.mixer.forward(x, batch, cache, state, own)
         x = torch.empty_like(x) if rounded else residual
         self.mixer_norm.add_normed(residual, own, first, next_out=x if rounded else None, clear=True)
-        second = self.feed_forward.forward(x, own)
-        self.ffn_norm.add_normed(residual, own, second, clear=True)
+        if self.ffn_norm is not None:
+            second = self.feed_forward.forward(x, own)
+            x = torch.empty_like(x) if rounded else residual
+            self.ffn_norm.add_normed(residual, own, second, next_out=x if rounded else None, clear=True)
+        if rounded:
+            batch.memo[ROUNDED_RESIDUAL] = x
         return None
 
     def parameters_bytes(self) -> int:

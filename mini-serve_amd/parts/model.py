@@ -9,7 +9,7 @@ from __future__ import annotations
 from dataclasses import dataclass
 
 from ..config.spec import ModelSpec
-from .base import KVNeed, Runtime, StateNeed, TensorSpec
+from .base import ROUNDED_RESIDUAL, KVNeed, Runtime, StateNeed, TensorSpec
 from .registry import part_class
 
 
@@ -143,7 +143,10 @@ class DecoderModel:
         for e in self.spec.run_order:
             cache = pool.view(e.cache, batch, e.writes_cache) if e.cache is not None else None
             state = pool.state_view(e.cache, batch) if e.cache is not None else None
+            left = batch.memo.get(ROUNDED_RESIDUAL)
             pending = self.blocks[e.layer].forward(residual, batch, cache, state, pending)
+            if left is not None and batch.memo.get(ROUNDED_RESIDUAL) is left:
+                del batch.memo[ROUNDED_RESIDUAL]  # an earlier block's copy: the stream has moved on since
         if batch.num_wanted == 0:
             return None
         x = self.final_norm.forward(residual, rows=batch.want_rows, add=pending)
