@@ -20,17 +20,12 @@
 #define PREP_MAX_DIM 1024
 #define PREP_PER_LANE (PREP_MAX_DIM / WAVE)
 
-// One element of a matrix that may exist as `splits` partial sums `stride` floats apart (added in ascending order).
-__device__ __forceinline__ float prep_read(const float* __restrict__ p, int splits, size_t stride) {
-  return splits == 1 ? *p : sum_splits(p, splits, stride);
-}
-
 template <typename T, typename TW>
 __global__ __launch_bounds__(256) void head_prepare_store_kernel(
-    const float* __restrict__ qkv, int ld, int splits, size_t stride, T* __restrict__ q_out, const int* __restrict__ slots,
-    const TW* __restrict__ qw, const TW* __restrict__ kw, int norm_order, float eps, const float* __restrict__ rope, int rot,
-    int pairing, const float* __restrict__ v_first, int v_first_ld, int first_splits, size_t first_stride, float blend,
-    T* __restrict__ kc, T* __restrict__ vc, int Hq, int Hkv, int D, int Dv, int page_size, int units) {
+    const float* __restrict__ qkv, int ld, T* __restrict__ q_out, const int* __restrict__ slots, const TW* __restrict__ qw,
+    const TW* __restrict__ kw, int norm_order, float eps, const float* __restrict__ rope, int rot, int pairing,
+    const float* __restrict__ v_first, int v_first_ld, float blend, T* __restrict__ kc, T* __restrict__ vc, int Hq, int Hkv,
+    int D, int Dv, int page_size, int units) {
   const int t = blockIdx.x, wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
   const int unit = blockIdx.y * 4 + wave;
   if (unit >= units) return;
@@ -42,8 +37,8 @@ __global__ __launch_bounds__(256) void head_prepare_store_kernel(
     const float* src = row + (size_t)Hq * D + (size_t)Hkv * D + (size_t)h * Dv;
     const float* first = v_first ? v_first + (size_t)t * v_first_ld + (size_t)h * Dv : nullptr;
     for (int d = lane; d < Dv; d += WAVE) {
-      float v = prep_read(src + d, splits, stride);
-      if (first) v = (1.f - blend) * v + blend * prep_read(first + d, first_splits, first_stride);
+      float v = src[d];
+      if (first) v = (1.f - blend) * v + blend * first[d];
       vc[((page * Hkv + h) * Dv + d) * page_size + off] = from_f32<T>(v);
     }
     return;
@@ -57,10 +52,7 @@ __global__ __launch_bounds__(256) void head_prepare_store_kernel(
   float pre = 1.f;
   if (norm_order == MS_NORM_BEFORE) {
     float ss = 0.f;
-    for (int d = lane; d < D; d += WAVE) {
-      const float x = prep_read(src + d, splits, stride);
-      ss += x * x;
-    }
+    for (int d = lane; d < D; d += WAVE) ss += src[d] * src[d];
     pre = 1.f / sqrtf(wave_sum(ss) / (float)D + eps);
   }
   const bool w_before = norm_order == MS_NORM_BEFORE && w != nullptr;
@@ -71,13 +63,13 @@ __global__ __launch_bounds__(256) void head_prepare_store_kernel(
     const int d = lane + i * WAVE;
     float v = 0.f;
     if (d < D) {
-      v = prep_read(src + d, splits, stride) * pre * (w_before ? to_f32(w[d]) : 1.f);
+      v = src[d] * pre * (w_before ? to_f32(w[d]) : 1.f);
       if (d < rot) {
         const bool adjacent = pairing == MS_ROPE_ADJACENT;
         const bool first = adjacent ? (d & 1) == 0 : d < half;
         const int j = adjacent ? d / 2 : (d < half ? d : d - half);
         const int pd = adjacent ? (d ^ 1) : (d < half ? d + half : d - half);
-        const float p = prep_read(src + pd, splits, stride) * pre * (w_before ? to_f32(w[pd]) : 1.f);
+        const float p = src[pd] * pre * (w_before ? to_f32(w[pd]) : 1.f);
         v = first ? v * cs[j] - p * cs[half + j] : v * cs[j] + p * cs[half + j];
       }
     }
@@ -97,17 +89,11 @@ __global__ __launch_bounds__(256) void head_prepare_store_kernel(
   }
 }
 
-// qkv and v_first may each exist as partial sums of a matrix product (`splits` slices `stride` floats apart, 1: the matrix
-// itself): the kernel adds them where it reads, so that a product over few rows needs no reduction kernel behind it.
-extern "C" int ms_head_prepare_store(const float* qkv, int ld, int splits, long long stride, void* q_out, int is_bf16,
-                                     const int* slots, const void* qw, const void* kw, int w_is_bf16, int norm_order, float eps,
-                                     const float* rope, int rot, int pairing, const float* v_first, int v_first_ld,
-                                     int first_splits, long long first_stride, float blend, void* kc, void* vc, int tokens, int Hq,
-                                     int Hkv, int D, int Dv, int page_size, hipStream_t st) {
+extern "C" int ms_head_prepare_store(const float* qkv, int ld, void* q_out, int is_bf16, const int* slots, const void* qw,
+                                     const void* kw, int w_is_bf16, int norm_order, float eps, const float* rope, int rot,
+                                     int pairing, const float* v_first, int v_first_ld, float blend, void* kc, void* vc,
+                                     int tokens, int Hq, int Hkv, int D, int Dv, int page_size, hipStream_t st) {
   if (tokens <= 0) return MS_OK;
-  if (splits < 1 || (splits > 1 && stride < (long long)tokens * ld) ||
-      (v_first != nullptr && (first_splits < 1 || (first_splits > 1 && first_stride < (long long)tokens * v_first_ld))))
-    return MS_BAD_ARG;
   if (qkv == nullptr || q_out == nullptr || Hq <= 0 || Hkv <= 0 || D <= 0 || Dv <= 0 || page_size <= 0 || rot < 0 || rot > D ||
       rot % 2 || (rot > 0) != (rope != nullptr) || ld < Hq * D + (slots ? Hkv * (D + Dv) : 0) ||
       (slots != nullptr && (kc == nullptr || vc == nullptr)) || !(eps >= 0.f) || tokens > 65535 * 32767 ||
@@ -121,7 +107,7 @@ extern "C" int ms_head_prepare_store(const float* qkv, int ld, int splits, long 
   const int units = slots ? Hq + 2 * Hkv : Hq;
   if ((units + 3) / 4 > 65535) return MS_BAD_ARG;
   const dim3 grid(tokens, (units + 3) / 4);
-#define PREP(T, TW) head_prepare_store_kernel<T, TW><<<grid, 256, 0, st>>>(qkv, ld, splits, (size_t)stride, (T*)q_out, slots, (const TW*)qw, (const TW*)kw, norm_order, eps, rope, rot, pairing, v_first, v_first_ld, first_splits, (size_t)first_stride, blend, (T*)kc, (T*)vc, Hq, Hkv, D, Dv, page_size, units)
+#define PREP(T, TW) head_prepare_store_kernel<T, TW><<<grid, 256, 0, st>>>(qkv, ld, (T*)q_out, slots, (const TW*)qw, (const TW*)kw, norm_order, eps, rope, rot, pairing, v_first, v_first_ld, blend, (T*)kc, (T*)vc, Hq, Hkv, D, Dv, page_size, units)
   if (is_bf16) { if (w_is_bf16) PREP(bf16, bf16); else PREP(bf16, float); }
   else { if (w_is_bf16) PREP(float, bf16); else PREP(float, float); }
 #undef PREP

@@ -96,9 +96,9 @@ _SIGNATURES = {
     "ms_sample_scratch_bytes": [_c_int],
     "ms_sample_rows_static": [_c_void, _c_int, _c_int, _c_ll, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void],
     "ms_sample_rows_static_max_rows": [],
-    "ms_head_prepare_store": [_c_void, _c_int, _c_int, _c_ll, _c_void, _c_int, _c_void, _c_void, _c_void, _c_int, _c_int, _c_float,
-                              _c_void, _c_int, _c_int, _c_void, _c_int, _c_int, _c_ll, _c_float, _c_void, _c_void, _c_int, _c_int,
-                              _c_int, _c_int, _c_int, _c_int, _c_void],
+    "ms_head_prepare_store": [_c_void, _c_int, _c_void, _c_int, _c_void, _c_void, _c_void, _c_int, _c_int, _c_float, _c_void, _c_int,
+                              _c_int, _c_void, _c_int, _c_float, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
+                              _c_void],
     "ms_moe_route": [_c_void, _c_int, _c_int, _c_ll, _c_void, _c_int, _c_int, _c_int, _c_int, _c_void, _c_void, _c_void],
     "ms_moe_plan": [_c_void, _c_int, _c_int, _c_int, _c_int, _c_void, _c_void, _c_void, _c_void, _c_void],
     "ms_moe_gemm": [_c_void, _c_int, _c_void, _c_void, _c_void, _c_int, _c_int, _c_void, _c_void, _c_void, _c_void, _c_void,
@@ -1232,57 +1232,20 @@ HEAD_NORMS = {None: 0, "before": 1, "after": 2}  # where a per-head RMS norm sit
 PREPARE_MAX_HEAD_DIM = 1024
 
 
-class SplitColumns:
-    """Columns ``start ..`` of a ``SplitSum``'s rows: what a view ``matrix[:, start:]`` is to a matrix."""
-
-    __slots__ = ("split", "start")
-
-    def __init__(self, split: SplitSum, start: int):
-        self.split, self.start = split, int(start)
-
-
-def _rows_or_sums(v, name: str, rows: int, least: int):
-    """``(pointer, row stride, splits, split stride)`` of float32 rows that are a matrix (possibly a view of wider rows),
-    a ``SplitSum`` or ``SplitColumns`` of one; at least ``least`` columns are needed."""
-    start = 0
-    if isinstance(v, SplitColumns):
-        v, start = v.split, v.start
-    if isinstance(v, SplitSum):
-        _dev(v.parts, name, F32, 3)
-        m, n = v.shape
-        if m != rows or n - start < least or start < 0:
-            raise ValueError(f"{name} is {v.shape} from column {start}; {rows} rows of at least {least} columns are needed")
-        return v.parts.data_ptr() + 4 * start, n, v.splits, v.stride
-    if not (isinstance(v, torch.Tensor) and v.is_cuda and v.dtype == F32 and v.dim() == 2 and v.stride(1) == 1):
-        raise TypeError(f"{name} must be float32 rows on the GPU with contiguous elements")
-    if v.shape[0] != rows or v.shape[1] < least:
-        raise ValueError(f"{name} is {tuple(v.shape)}; {rows} rows of at least {least} columns are needed")
-    return v.data_ptr(), v.stride(0), 1, 0
-
-
 def head_prepare_store(qkv, slots, norm: str | None, q_weight, k_weight, eps, rope, pairing, k_cache, v_cache, num_heads,
                        num_kv_heads, head_dim, value_dim, out_dtype, v_first=None, blend: float = 0.0) -> torch.Tensor:
     """From float32 ``qkv [T, Hq D + Hkv D + Hkv Dv]``: rotation of the first ``rope.shape[1]`` elements of each query and
     key head, in pairs as ``pairing`` names them, by the angles of ``rope`` (a ``rope_table`` of these tokens; None: no
     rotation), and an RMS norm per head, ``norm="before"`` the rotation or ``"after"`` it (weights ``[D]`` each, or None for
-    a bare division by the root mean square; ``norm=None``: no norm). ``v_first`` (float32 rows of at least ``Hkv Dv``
-    columns, one per token, possibly a view of wider rows): the values become ``(1 - blend) v + blend v_first``. Keys
+    a bare division by the root mean square; ``norm=None``: no norm). ``v_first`` (a float32 tensor of at least ``Hkv Dv``
+    columns, one row per token, possibly a view of wider rows): the values become ``(1 - blend) v + blend v_first``. Keys
     and values are stored into the cache pages at ``slots`` (skipped when ``slots`` is None). Returns the finished queries
-    ``[T, Hq D]`` in ``out_dtype``. ``qkv`` may be a ``SplitSum`` and ``v_first`` a ``SplitSum`` or ``SplitColumns``: the
-    kernel adds the partial sums where it reads them."""
+    ``[T, Hq D]`` in ``out_dtype``."""
+    _dev(qkv, "qkv", F32, 2)
+    t = qkv.shape[0]
     width = num_heads * head_dim + num_kv_heads * (head_dim + value_dim)
-    if isinstance(qkv, SplitSum):
-        t = qkv.shape[0]
-        if qkv.shape[1] != width:
-            raise ValueError(f"qkv has width {qkv.shape[1]}, expected {width}")
-        device = qkv.parts.device
-    else:
-        _dev(qkv, "qkv", F32, 2)
-        t = qkv.shape[0]
-        if qkv.shape[1] != width:
-            raise ValueError(f"qkv has width {qkv.shape[1]}, expected {width}")
-        device = qkv.device
-    q_ptr, q_ld, q_splits, q_stride = _rows_or_sums(qkv, "qkv", t, width)
+    if qkv.shape[1] != width:
+        raise ValueError(f"qkv has width {qkv.shape[1]}, expected {width}")
     if out_dtype not in (F32, BF16):
         raise TypeError(f"unsupported output dtype {out_dtype}")
     if norm not in HEAD_NORMS:
@@ -1312,11 +1275,18 @@ def head_prepare_store(qkv, slots, norm: str | None, q_weight, k_weight, eps, ro
         rot_dim = rope.shape[1]
         if rope.shape[0] != t or rot_dim % 2 or rot_dim > head_dim or rot_dim < 2:
             raise ValueError(f"rotation table is {tuple(rope.shape)}; {t} tokens and an even width up to {head_dim} are needed")
-    f_ptr, f_ld, f_splits, f_stride = (None, 0, 1, 0) if v_first is None else _rows_or_sums(v_first, "v_first", t, num_kv_heads * value_dim)
-    q_out = torch.empty((t, num_heads * head_dim), dtype=out_dtype, device=device)
+    first_ld = 0
+    if v_first is not None:
+        if not (isinstance(v_first, torch.Tensor) and v_first.is_cuda and v_first.dtype == F32 and v_first.dim() == 2
+                and v_first.stride(1) == 1):
+            raise TypeError("v_first must be float32 rows on the GPU with contiguous elements")
+        if v_first.shape[0] != t or v_first.shape[1] < num_kv_heads * value_dim:
+            raise ValueError(f"v_first is {tuple(v_first.shape)}; {t} rows of at least {num_kv_heads * value_dim} values are needed")
+        first_ld = v_first.stride(0)
+    q_out = torch.empty((t, num_heads * head_dim), dtype=out_dtype, device=qkv.device)
     _check(library().ms_head_prepare_store(
-        q_ptr, q_ld, q_splits, q_stride, q_out.data_ptr(), int(out_dtype == BF16), _ptr(slots), _ptr(q_weight), _ptr(k_weight), w_bf16,
-        HEAD_NORMS[norm], float(eps), _ptr(rope), int(rot_dim), pair, f_ptr, int(f_ld), int(f_splits), int(f_stride), float(blend),
+        qkv.data_ptr(), qkv.shape[1], q_out.data_ptr(), int(out_dtype == BF16), _ptr(slots), _ptr(q_weight), _ptr(k_weight), w_bf16,
+        HEAD_NORMS[norm], float(eps), _ptr(rope), int(rot_dim), pair, _ptr(v_first), int(first_ld), float(blend),
         _ptr(k_cache) if slots is not None else None, _ptr(v_cache) if slots is not None else None, t, num_heads, num_kv_heads,
         head_dim, int(value_dim), page_size, _stream()), "head_prepare_store")
     return q_out

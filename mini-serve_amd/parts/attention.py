@@ -190,24 +190,21 @@ class GQAttention(Mixer):
 
     def _forward_prepared(self, x, batch, cache, residual, table, pairing, eps):
         ops = self.rt.ops
-        # what norms and blends read is not rounded; over few rows the product leaves partial sums, which the preparation adds
-        qkv = ops.linear(x, self.qkv, out_dtype=torch.float32, defer=True)
+        qkv = ops.linear(x, self.qkv, out_dtype=torch.float32)  # what norms and blends read is not rounded
         v_first = None
         if self.value_blend is not None:
             if not cache.writes:
                 raise NotImplementedError("a layer that blends values keeps keys and values of its own")
             if self.value_blend == "first":
                 # a view of this step's projection: the values as projected, one row per token
-                at = (self.heads + self.kv_heads) * self.head_dim
-                batch.memo[self.blend_key] = ops.SplitColumns(qkv, at) if isinstance(qkv, ops.SplitSum) else qkv[:, at:]
+                batch.memo[self.blend_key] = qkv[:, (self.heads + self.kv_heads) * self.head_dim:]
             else:
                 v_first = batch.memo.get(self.blend_key)
                 if v_first is None:
                     raise ValueError(f"no earlier layer of the step kept values for {self.blend_key[1]!r}")
-                kept = v_first.split.shape[1] - v_first.start if isinstance(v_first, ops.SplitColumns) else v_first.shape[1]
-                if kept != self.kv_heads * self.value_dim:
+                if v_first.shape[1] != self.kv_heads * self.value_dim:
                     raise ValueError(f"values of width {self.kv_heads * self.value_dim} cannot be blended with kept values of "
-                                     f"width {kept}")
+                                     f"width {v_first.shape[1]}")
         norm = None if self.qk_norm_eps is None else ("after" if self.qk_norm == "head_rotated" else "before")
         q = ops.head_prepare_store(qkv, cache.slots if cache.writes else None, norm, self.q_norm, self.k_norm, eps, table, pairing,
                                    cache.k, cache.v, self.heads, self.kv_heads, self.head_dim, self.value_dim, self.rt.dtype,

@@ -161,18 +161,6 @@ def test_rotation_norm_blend_and_store(hq, hk, d, e, rot, order, weights, blend,
     close(vc.permute(0, 3, 1, 2).reshape(-1, hk, e)[at], v, dtype, "values", tol)
     untouched = np.setdiff1d(np.arange(5 * PAGE), slots)
     assert not kc.permute(0, 2, 1, 3).reshape(-1, hk * d)[dev(untouched, torch.int64)].any()
-    # the projection (and the first values) as partial sums of a product over few rows: the kernel adds them itself
-    def in_parts(a, n=3):
-        parts = rng.normal(size=(n - 1,) + a.shape).astype(np.float32)
-        last = (a - parts.astype(np.float64).sum(0)).astype(np.float32)
-        return o.SplitSum(dev(np.concatenate([parts, last[None]])))
-    kc2, vc2 = torch.zeros_like(kc), torch.zeros_like(vc)
-    got2 = o.head_prepare_store(in_parts(x), dev(slots, torch.int32), order, None if qw is None else dev(qw), None if kw is None else dev(kw),
-                                eps, rope_for(o, pos, rot), rot[3] if rot else "halves", kc2, vc2, hq, hk, d, e, dtype,
-                                o.SplitColumns(in_parts(wide, 5), 5) if blend else None, lam)
-    close(got2, q.reshape(T, -1), dtype, "queries from partial sums", tol)
-    close(kc2.permute(0, 2, 1, 3).reshape(-1, hk, d)[at], k, dtype, "keys from partial sums", tol)
-    close(vc2.permute(0, 3, 1, 2).reshape(-1, hk, e)[at], v, dtype, "values from partial sums", tol)
     # a layer that keeps nothing: queries only, the cache stays as it is
     before = kc.clone()
     again = o.head_prepare_store(dev(x), None, order, None if qw is None else dev(qw), None if kw is None else dev(kw), eps,
