@@ -12,10 +12,12 @@ from .qwen3 import Qwen3Config
 from .kakunex import KakunexConfig
 from .fimolix import FimolixConfig
 from .reselorn import ReselornConfig
+from .zigelorn import ZigelornConfig
 from .presets import PRESETS, preset
 
 __all__ = [
     "ARCHITECTURES", "architecture_name", "config_from_dict", "load_config", "load_config_dict",
     "register_architecture", "unregister_architecture", "LayerSpec", "ModelSpec", "PartSpec",
-    "RunEntry", "Qwen3Config", "KakunexConfig", "FimolixConfig", "ReselornConfig", "PRESETS", "preset",
+    "RunEntry", "Qwen3Config", "KakunexConfig", "FimolixConfig", "ReselornConfig", "ZigelornConfig",
+    "PRESETS", "preset",
 ]

@@ -1,5 +1,7 @@
-// A mixture of gated feed-forward experts: routing, a plan that sorts the step's (token, chosen expert) pairs by expert,
-// the two products per expert over the sorted pairs, and the weighted sum back into the stream.
+// A mixture of feed-forward experts (gated, act(gate x) * up x, or plain, act(up x)): routing, a plan that sorts the step's
+// (token, chosen expert) pairs by expert, the two products per expert over the sorted pairs, and the weighted sum back
+// into the stream. Router outputs from `real` on are identity experts: they have no weights, their pairs are left out of
+// the plan, and the weighted sum adds the token's own input for them.
 //
 // A step of T tokens that each choose `top` of E experts has P = T top pairs; pair p = t * top + j is token t's j-th
 // choice (largest logit first). The plan cuts every expert's run of pairs into tiles of `tile_rows` pairs; the product
@@ -74,9 +76,132 @@ extern "C" int ms_moe_route(const float* logits, int ld, int splits, long long s
 }
 
 // ---------------------------------------------------------------------------------------------
+// Routing by scores: s = softmax(logits[t]) over all E outputs; the choice is made by c = s + correction (correction may
+// be absent), the weights are the chosen outputs' s as they stand (not renormalised). With groups > 1 the E outputs form
+// `groups` equal groups of neighbours, a group's score is its largest c, and only outputs of the `keep` best groups
+// (ties: the lower group) can be chosen: the others' c counts as minus infinity. The `top` largest c are chosen, largest
+// first (ties: the lower index). One wave per token; s and c of a token pass through the wave's own rows of LDS.
+template <typename TB>
+__global__ __launch_bounds__(256) void moe_route_scored_kernel(const float* __restrict__ logits, int ld, int splits, size_t stride,
+                                                               const TB* __restrict__ correction, int T, int E, int top,
+                                                               int groups, int keep, int* __restrict__ ids,
+                                                               float* __restrict__ weights) {
+  __shared__ float ss[4][MOE_MAX_EXPERTS], cs[4][MOE_MAX_EXPERTS];
+  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+  const int t = blockIdx.x * 4 + wave;
+  const bool live = t < T;  // every wave stays for the block's barriers
+  float c[MOE_MAX_EXPERTS / WAVE];
+  float m = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < MOE_MAX_EXPERTS / WAVE; ++i) {
+    const int e = lane + i * WAVE;
+    c[i] = (live && e < E) ? sum_splits(logits + (size_t)t * ld + e, splits, stride) : -INFINITY;
+    m = fmaxf(m, c[i]);
+  }
+  m = wave_max(m);
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < MOE_MAX_EXPERTS / WAVE; ++i) {
+    c[i] = lane + i * WAVE < E ? expf(c[i] - m) : 0.f;
+    sum += c[i];
+  }
+  sum = wave_sum(sum);
+#pragma unroll
+  for (int i = 0; i < MOE_MAX_EXPERTS / WAVE; ++i) {
+    const int e = lane + i * WAVE;
+    if (e < E) {
+      const float sc = c[i] / sum;
+      ss[wave][e] = sc;
+      c[i] = sc + (correction ? to_f32(correction[e]) : 0.f);
+      cs[wave][e] = c[i];
+    } else {
+      c[i] = -INFINITY;
+    }
+  }
+  if (groups > 1) {
+    const int n = E / groups;
+    __syncthreads();
+    float gm[MOE_MAX_EXPERTS / WAVE];  // lane l holds the scores of groups l, l + 64, ...
+    bool taken[MOE_MAX_EXPERTS / WAVE];
+#pragma unroll
+    for (int i = 0; i < MOE_MAX_EXPERTS / WAVE; ++i) {
+      const int g = lane + i * WAVE;
+      gm[i] = -INFINITY;
+      taken[i] = false;
+      if (g < groups)
+        for (int k = 0; k < n; ++k) gm[i] = fmaxf(gm[i], cs[wave][g * n + k]);
+    }
+    __syncthreads();  // cs is read; from here on it says which groups stay (1) and which do not (0)
+#pragma unroll
+    for (int i = 0; i < MOE_MAX_EXPERTS / WAVE; ++i)
+      if (lane + i * WAVE < groups) cs[wave][lane + i * WAVE] = 0.f;
+    for (int j = 0; j < keep; ++j) {
+      float best = -INFINITY;
+      int at = 0x7fffffff;
+#pragma unroll
+      for (int i = 0; i < MOE_MAX_EXPERTS / WAVE; ++i)
+        if (lane + i * WAVE < groups && !taken[i] && (at == 0x7fffffff || gm[i] > best)) { best = gm[i]; at = lane + i * WAVE; }
+#pragma unroll
+      for (int off = WAVE / 2; off > 0; off >>= 1) {
+        const float ob = __shfl_xor(best, off, WAVE);
+        const int oa = __shfl_xor(at, off, WAVE);
+        if (oa != 0x7fffffff && (at == 0x7fffffff || ob > best || (ob == best && oa < at))) { best = ob; at = oa; }
+      }
+#pragma unroll
+      for (int i = 0; i < MOE_MAX_EXPERTS / WAVE; ++i)
+        if (lane + i * WAVE == at) { taken[i] = true; cs[wave][at] = 1.f; }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < MOE_MAX_EXPERTS / WAVE; ++i) {
+      const int e = lane + i * WAVE;
+      if (e < E && cs[wave][e / n] == 0.f) c[i] = -INFINITY;
+    }
+  } else {
+    __syncthreads();
+  }
+  if (!live) return;
+  for (int j = 0; j < top; ++j) {
+    float best = -INFINITY;
+    int at = 0x7fffffff;
+#pragma unroll
+    for (int i = 0; i < MOE_MAX_EXPERTS / WAVE; ++i)
+      if (c[i] > best) { best = c[i]; at = lane + i * WAVE; }
+#pragma unroll
+    for (int off = WAVE / 2; off > 0; off >>= 1) {
+      const float ob = __shfl_xor(best, off, WAVE);
+      const int oa = __shfl_xor(at, off, WAVE);
+      if (ob > best || (ob == best && oa < at)) { best = ob; at = oa; }
+    }
+    if (at >= E) at = j;  // nothing left to choose by (no numbers, or fewer outputs in the kept groups than choices)
+#pragma unroll
+    for (int i = 0; i < MOE_MAX_EXPERTS / WAVE; ++i)
+      if (lane + i * WAVE == at) c[i] = -INFINITY;
+    if (lane == 0) {
+      ids[(size_t)t * top + j] = at;
+      weights[(size_t)t * top + j] = ss[wave][at];
+    }
+  }
+}
+
+extern "C" int ms_moe_route_scored(const float* logits, int ld, int splits, long long stride, const void* correction,
+                                   int correction_is_bf16, int T, int E, int top, int groups, int keep, int* ids, float* weights,
+                                   hipStream_t st) {
+  if (T <= 0) return MS_OK;
+  if (logits == nullptr || ids == nullptr || weights == nullptr || E < 1 || top < 1 || top > E || ld < E || splits < 1 ||
+      (splits > 1 && stride < (long long)T * ld) || groups < 1 || E % groups || keep < 1 || keep > groups)
+    return MS_BAD_ARG;
+  if (E > MOE_MAX_EXPERTS || top > MOE_MAX_TOP) return MS_UNSUPPORTED;
+  const unsigned blocks = (unsigned)((T + 3) / 4);
+  if (correction_is_bf16) moe_route_scored_kernel<bf16><<<blocks, 256, 0, st>>>(logits, ld, splits, (size_t)stride, (const bf16*)correction, T, E, top, groups, keep, ids, weights);
+  else moe_route_scored_kernel<float><<<blocks, 256, 0, st>>>(logits, ld, splits, (size_t)stride, (const float*)correction, T, E, top, groups, keep, ids, weights);
+  return launch_status();
+}
+
+// ---------------------------------------------------------------------------------------------
 // The plan, one block: counts per expert, every expert's run of `order` (order[i] = the pair at sorted place i), and the
 // tiles: tile n covers places tile_start[n] .. tile_start[n] + tile_count[n] - 1 of expert tile_expert[n]. Tiles past the
-// last get a count of zero.
+// last get a count of zero. Pairs whose id is E or more (identity experts) are in no run and no tile.
 __global__ __launch_bounds__(1024) void moe_plan_kernel(const int* __restrict__ ids, int P, int E, int tile_rows, int max_tiles,
                                                         int* __restrict__ order, int* __restrict__ tile_expert,
                                                         int* __restrict__ tile_start, int* __restrict__ tile_count) {
@@ -85,7 +210,8 @@ __global__ __launch_bounds__(1024) void moe_plan_kernel(const int* __restrict__ 
   const int tid = threadIdx.x;
   for (int e = tid; e < E; e += 1024) { counts[e] = 0; cursor[e] = 0; }
   __syncthreads();
-  for (int p = tid; p < P; p += 1024) atomicAdd(&counts[min(max(ids[p], 0), E - 1)], 1);
+  for (int p = tid; p < P; p += 1024)
+    if (ids[p] < E) atomicAdd(&counts[max(ids[p], 0)], 1);
   __syncthreads();
   if (tid == 0) {
     int off = 0, nt = 0;
@@ -114,7 +240,8 @@ __global__ __launch_bounds__(1024) void moe_plan_kernel(const int* __restrict__ 
     tile_count[n] = 0;
   }
   for (int p = tid; p < P; p += 1024) {
-    const int e = min(max(ids[p], 0), E - 1);
+    if (ids[p] >= E) continue;
+    const int e = max(ids[p], 0);
     order[offsets[e] + atomicAdd(&cursor[e], 1)] = p;
   }
 }
@@ -136,9 +263,10 @@ extern "C" int ms_moe_plan(const int* ids, int P, int E, int tile_rows, int max_
 // pairs by rows (NT = 4: 64 columns a block), a tile of 16 pairs by columns (64 NT columns a block: steps of few tokens,
 // where every chosen expert has a tile of its own and its weights are streamed once; the fewer tiles the step can have,
 // the narrower the waves' runs of columns, so that the chip still gets waves enough to stream with).
-//   GATED: rows are x[token of the pair] (K = the model's width), two weights per expert, gate and up [E, N, K]; the result
-//          act(gate) * up goes to h[sorted place][N] in the compute type.
-//   else:  rows are h[sorted place] (K = the experts' width), one weight per expert [E, N, K]; the result times the pair's
+//   MODE 1 (gated): rows are x[token of the pair] (K = the model's width), two weights per expert, gate and up [E, N, K];
+//          the result act(gate) * up goes to h[sorted place][N] in the compute type.
+//   MODE 2 (plain first product): the same rows, one weight per expert; act(up) goes to h[sorted place][N].
+//   MODE 0: rows are h[sorted place] (K = the experts' width), one weight per expert [E, N, K]; the result times the pair's
 //          routing weight goes to y[pair][N] in float32.
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 moe_bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float moe_floatx4;
@@ -158,11 +286,12 @@ template <bool ALIGNED> __device__ __forceinline__ moe_bf16x8 moe_load(const bf1
   return x.v;
 }
 
-template <bool GATED, bool ALIGNED, int NT, bool KSPLIT = false>
+template <int MODE, bool ALIGNED, int NT, bool KSPLIT = false>
 __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(
     const bf16* __restrict__ a, int lda, const bf16* __restrict__ w1, const bf16* __restrict__ w2, void* __restrict__ out,
     const int* __restrict__ order, const int* __restrict__ tile_expert, const int* __restrict__ tile_start,
     const int* __restrict__ tile_count, const float* __restrict__ pair_weight, int top, int N, int K, int tile_rows, int act) {
+  constexpr bool GATED = MODE == 1, FIRST = MODE != 0;
   const int count = tile_count[blockIdx.x];
   if (count == 0) return;
   const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE, l16 = lane % 16, grp = lane / 16;
@@ -178,7 +307,7 @@ __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(
   const int e = tile_expert[blockIdx.x], start = tile_start[blockIdx.x];
   const bool row_ok = m0 + l16 < count;
   const int place = start + m0 + (row_ok ? l16 : 0);
-  const bf16* ap = a + (size_t)(GATED ? order[place] / top : place) * lda;
+  const bf16* ap = a + (size_t)(FIRST ? order[place] / top : place) * lda;
   const bf16* wp1[NT];
   const bf16* wp2[NT];
   bool col_ok[NT];
@@ -248,6 +377,11 @@ __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt)
         if (col_ok[nt]) o[nt * 16] = static_cast<bf16>(gated_value(acc1[nt][r], acc2[nt][r], act, 0.f));
+    } else if (FIRST) {
+      bf16* o = (bf16*)out + (size_t)(start + m) * N + n0 + l16;
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+        if (col_ok[nt]) o[nt * 16] = static_cast<bf16>(activate(acc1[nt][r], act));
     } else {
       const int pair = order[start + m];
       const float pw = pair_weight[pair];
@@ -273,11 +407,12 @@ template <int N_> __device__ __forceinline__ void moe_wait_loads() {
   __builtin_amdgcn_s_waitcnt((N_ & 15) | ((N_ >> 4) << 14) | (7 << 4) | (15 << 8));  // vmcnt alone
 }
 
-template <bool GATED, int BM, int WR, int WC>
+template <int MODE, int BM, int WR, int WC>
 __global__ __launch_bounds__(256, 2) void moe_gemm_bf16_lds_kernel(
     const bf16* __restrict__ a, int lda, const bf16* __restrict__ w1, const bf16* __restrict__ w2, void* __restrict__ out,
     const int* __restrict__ order, const int* __restrict__ tile_expert, const int* __restrict__ tile_start,
     const int* __restrict__ tile_count, const float* __restrict__ pair_weight, int top, int N, int K, int act) {
+  constexpr bool GATED = MODE == 1, FIRST = MODE != 0;
   static_assert(WR * WC == 4, "four waves a block");
   constexpr int BN = 128, KS = 64, STAGES = 2;
   constexpr int WM = BM / WR, WN = BN / WC, FM = WM / 16, FN = WN / 16;
@@ -303,7 +438,7 @@ __global__ __launch_bounds__(256, 2) void moe_gemm_bf16_lds_kernel(
   for (int j = 0; j < XI; ++j) {
     const int R = (wave * XI + j) * RPI + lrow;
     const int place = start + min(R, count - 1);
-    xsrc[j] = a + (size_t)(GATED ? order[place] / top : place) * lda + ((lslot ^ ((R >> 1) & (CPR - 1))) * 8);
+    xsrc[j] = a + (size_t)(FIRST ? order[place] / top : place) * lda + ((lslot ^ ((R >> 1) & (CPR - 1))) * 8);
   }
 #pragma unroll
   for (int j = 0; j < WI; ++j) {
@@ -383,6 +518,20 @@ __global__ __launch_bounds__(256, 2) void moe_gemm_bf16_lds_kernel(
           for (int c = 0; c < 4; ++c)
             if (col + c < N) o[col + c] = q.v[c];
       }
+    } else if (FIRST) {
+      bf16* o = (bf16*)out + (size_t)(start + m) * N;
+#pragma unroll
+      for (int i = 0; i < FN; ++i) {
+        const int col = n0 + wn + i * 16 + g * 4;
+        union { uint2 u; bf16 v[4]; } q;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) q.v[c] = static_cast<bf16>(activate(acc[i][j][c], act));
+        if (vec && col + 3 < N) *reinterpret_cast<uint2*>(o + col) = q.u;
+        else
+#pragma unroll
+          for (int c = 0; c < 4; ++c)
+            if (col + c < N) o[col + c] = q.v[c];
+      }
     } else {
       const int pair = order[start + m];
       const float pw = pair_weight[pair];
@@ -400,33 +549,34 @@ __global__ __launch_bounds__(256, 2) void moe_gemm_bf16_lds_kernel(
   }
 }
 
-template <bool GATED, int BM, int WR, int WC>
+template <int MODE, int BM, int WR, int WC>
 static int moe_launch_lds(const void* a, int lda, const void* w1, const void* w2, void* out, const int* order, const int* tile_expert,
                           const int* tile_start, const int* tile_count, const float* pair_weight, int max_tiles, int top, int N,
                           int K, int act, hipStream_t st) {
   constexpr int lds_bytes = 2 * (BM + 128) * 128;
   static bool ready = false;  // more than 48 KB of LDS is asked for once per kernel
   if (!ready) {
-    if (hipFuncSetAttribute((const void*)moe_gemm_bf16_lds_kernel<GATED, BM, WR, WC>, hipFuncAttributeMaxDynamicSharedMemorySize,
+    if (hipFuncSetAttribute((const void*)moe_gemm_bf16_lds_kernel<MODE, BM, WR, WC>, hipFuncAttributeMaxDynamicSharedMemorySize,
                             lds_bytes) != hipSuccess)
       return MS_LAUNCH_FAILED;
     ready = true;
   }
-  const int cols = GATED ? 64 : 128;
+  const int cols = MODE == 1 ? 64 : 128;
   const dim3 grid((N + cols - 1) / cols, max_tiles);
   if (grid.y > 65535) return MS_BAD_ARG;
-  moe_gemm_bf16_lds_kernel<GATED, BM, WR, WC><<<grid, 256, lds_bytes, st>>>((const bf16*)a, lda, (const bf16*)w1, (const bf16*)w2, out, order,
+  moe_gemm_bf16_lds_kernel<MODE, BM, WR, WC><<<grid, 256, lds_bytes, st>>>((const bf16*)a, lda, (const bf16*)w1, (const bf16*)w2, out, order,
                                                                            tile_expert, tile_start, tile_count, pair_weight, top, N, K, act);
   return launch_status();
 }
 
 // The same two products in true float32 on the vector units: 64 x 64 tiles through LDS, every output element one chain of
 // fused multiply-adds over k in ascending order.
-template <bool GATED>
+template <int MODE>
 __global__ __launch_bounds__(256) void moe_gemm_f32_kernel(
     const float* __restrict__ a, int lda, const float* __restrict__ w1, const float* __restrict__ w2, float* __restrict__ out,
     const int* __restrict__ order, const int* __restrict__ tile_expert, const int* __restrict__ tile_start,
     const int* __restrict__ tile_count, const float* __restrict__ pair_weight, int top, int N, int K, int act) {
+  constexpr bool GATED = MODE == 1, FIRST = MODE != 0;
   const int count = tile_count[blockIdx.x];
   if (count == 0) return;
   __shared__ float As[16][64 + 4];
@@ -438,7 +588,7 @@ __global__ __launch_bounds__(256) void moe_gemm_f32_kernel(
   const int tx = tid % 16, ty = tid / 16;      // 16 x 16 threads, 4 x 4 outputs each
   const int lr = tid / 4, lk = (tid % 4) * 4;  // loader: row within the tile, k offset
   const bool a_ok = lr < count;
-  const float* arow = a + (size_t)(a_ok ? (GATED ? order[start + lr] / top : start + lr) : 0) * lda;
+  const float* arow = a + (size_t)(a_ok ? (FIRST ? order[start + lr] / top : start + lr) : 0) * lda;
   const bool w_ok = n0 + lr < N;
   const size_t wat = ((size_t)e * N + (w_ok ? n0 + lr : 0)) * K;
   float acc1[4][4], acc2[4][4];
@@ -486,36 +636,39 @@ __global__ __launch_bounds__(256) void moe_gemm_f32_kernel(
   for (int i = 0; i < 4; ++i) {
     const int m = ty * 4 + i;
     if (m >= count) continue;
-    const int pair = GATED ? 0 : order[start + m];
-    const float pw = GATED ? 1.f : pair_weight[pair];
+    const int pair = FIRST ? 0 : order[start + m];
+    const float pw = FIRST ? 1.f : pair_weight[pair];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int n = n0 + tx * 4 + j;
       if (n >= N) continue;
       if (GATED) out[(size_t)(start + m) * N + n] = gated_value(acc1[i][j], acc2[i][j], act, 0.f);
+      else if (FIRST) out[(size_t)(start + m) * N + n] = activate(acc1[i][j], act);
       else out[(size_t)pair * N + n] = acc1[i][j] * pw;
     }
   }
 }
 
-// a: the rows ([tokens, lda] for the gated product, [P, lda] sorted places for the other); w1 (and w2, gated): [E, N, K];
-// out: h [P, N] (gated, the compute type) or y [P, N] float32. tile_rows: 16, 64 or 128 in bfloat16 (128: K a multiple of
-// 64 and 16-byte aligned rows), 64 in float32.
-extern "C" int ms_moe_gemm(const void* a, int lda, const void* w1, const void* w2, void* out, int is_bf16, int gated,
+// a: the rows ([tokens, lda] for a first product, [P, lda] sorted places for the second); w1 (and w2, gated): [E, N, K];
+// out: h [P, N] (a first product, the compute type) or y [P, N] float32. mode: 0 the second product, 1 the gated first
+// product, 2 the plain first product. tile_rows: 16, 64 or 128 in bfloat16 (128: K a multiple of 64 and 16-byte aligned
+// rows), 64 in float32.
+extern "C" int ms_moe_gemm(const void* a, int lda, const void* w1, const void* w2, void* out, int is_bf16, int mode,
                            const int* order, const int* tile_expert, const int* tile_start, const int* tile_count,
                            const float* pair_weight, int max_tiles, int top, int N, int K, int tile_rows, int act, hipStream_t st) {
   if (max_tiles <= 0 || N <= 0) return MS_OK;
-  if (a == nullptr || w1 == nullptr || (gated && w2 == nullptr) || out == nullptr || order == nullptr || tile_expert == nullptr ||
-      tile_start == nullptr || tile_count == nullptr || (!gated && pair_weight == nullptr) || top < 1 || K <= 0 || lda < K ||
-      act < 0 || act >= MS_ACT_COUNT)
+  const bool gated = mode == 1;
+  if (mode < 0 || mode > 2 || a == nullptr || w1 == nullptr || (gated && w2 == nullptr) || out == nullptr || order == nullptr ||
+      tile_expert == nullptr || tile_start == nullptr || tile_count == nullptr || (mode == 0 && pair_weight == nullptr) || top < 1 ||
+      K <= 0 || lda < K || (gated && (act < 0 || act >= MS_ACT_COUNT)) || (mode == 2 && !ms_act_ungated_ok(act)))
     return MS_BAD_ARG;
   if (is_bf16) {
     if (tile_rows != 16 && tile_rows != 64 && tile_rows != 128) return MS_BAD_ARG;
     const bool rows16 = (size_t)a % 16 == 0 && (size_t)w1 % 16 == 0 && (!gated || (size_t)w2 % 16 == 0) && lda % 8 == 0;
-    if (tile_rows >= 64 && K % 64 == 0 && rows16 && (gated || (size_t)out % 16 == 0)) {
+    if (tile_rows >= 64 && K % 64 == 0 && rows16 && (mode != 0 || (size_t)out % 16 == 0)) {
 #define MOE_LDS(G, BM, WR, WC) moe_launch_lds<G, BM, WR, WC>(a, lda, w1, w2, out, order, tile_expert, tile_start, tile_count, pair_weight, max_tiles, top, N, K, act, st)
-      if (tile_rows == 128) return gated ? MOE_LDS(true, 128, 2, 2) : MOE_LDS(false, 128, 2, 2);
-      return gated ? MOE_LDS(true, 64, 1, 4) : MOE_LDS(false, 64, 1, 4);
+      if (tile_rows == 128) return mode == 1 ? MOE_LDS(1, 128, 2, 2) : (mode == 2 ? MOE_LDS(2, 128, 2, 2) : MOE_LDS(0, 128, 2, 2));
+      return mode == 1 ? MOE_LDS(1, 64, 1, 4) : (mode == 2 ? MOE_LDS(2, 64, 1, 4) : MOE_LDS(0, 64, 1, 4));
 #undef MOE_LDS
     }
     if (tile_rows == 128) return MS_UNSUPPORTED;  // the caller plans tiles of 128 only where the kernel above takes them
@@ -527,46 +680,66 @@ extern "C" int ms_moe_gemm(const void* a, int lda, const void* w1, const void* w
       while (nt > 1 && busy * ((N + 64 * nt - 1) / (64 * nt)) < 1024) nt /= 2;
     }
     const bool aligned = K % 8 == 0 && lda % 8 == 0 && (size_t)a % 16 == 0 && (size_t)w1 % 16 == 0 && (!gated || (size_t)w2 % 16 == 0);
+#define MOE_ARGS (const bf16*)a, lda, (const bf16*)w1, (const bf16*)w2, out, order, tile_expert, tile_start, tile_count, pair_weight, top, N, K, tile_rows, act
     // still few blocks at the narrowest columns: the waves of a block share 16 columns and split K
     if (tile_rows == 16 && nt == 1 && aligned && K >= 512 && (max_tiles / 2 + 1) * ((N + 63) / 64) < 2048 && (N + 15) / 16 <= 65535) {
       const dim3 grid(max_tiles, (N + 15) / 16);
-      if (gated) moe_gemm_bf16_kernel<true, true, 1, true><<<grid, 256, 0, st>>>((const bf16*)a, lda, (const bf16*)w1, (const bf16*)w2, out, order, tile_expert, tile_start, tile_count, pair_weight, top, N, K, tile_rows, act);
-      else moe_gemm_bf16_kernel<false, true, 1, true><<<grid, 256, 0, st>>>((const bf16*)a, lda, (const bf16*)w1, (const bf16*)w2, out, order, tile_expert, tile_start, tile_count, pair_weight, top, N, K, tile_rows, act);
+      if (mode == 1) moe_gemm_bf16_kernel<1, true, 1, true><<<grid, 256, 0, st>>>(MOE_ARGS);
+      else if (mode == 2) moe_gemm_bf16_kernel<2, true, 1, true><<<grid, 256, 0, st>>>(MOE_ARGS);
+      else moe_gemm_bf16_kernel<0, true, 1, true><<<grid, 256, 0, st>>>(MOE_ARGS);
       return launch_status();
     }
     const int cols = tile_rows == 64 ? 64 : 64 * nt;
     const dim3 grid(max_tiles, (N + cols - 1) / cols);
     if (grid.y > 65535) return MS_BAD_ARG;
-#define MOE(G, A, T) moe_gemm_bf16_kernel<G, A, T><<<grid, 256, 0, st>>>((const bf16*)a, lda, (const bf16*)w1, (const bf16*)w2, out, order, tile_expert, tile_start, tile_count, pair_weight, top, N, K, tile_rows, act)
+#define MOE(G, A, T) moe_gemm_bf16_kernel<G, A, T><<<grid, 256, 0, st>>>(MOE_ARGS)
 #define MOE_NT(G, A) do { if (nt == 4) MOE(G, A, 4); else if (nt == 2) MOE(G, A, 2); else MOE(G, A, 1); } while (0)
-    if (gated) { if (aligned) MOE_NT(true, true); else MOE_NT(true, false); }
-    else { if (aligned) MOE_NT(false, true); else MOE_NT(false, false); }
+#define MOE_AL(G) do { if (aligned) MOE_NT(G, true); else MOE_NT(G, false); } while (0)
+    if (mode == 1) MOE_AL(1);
+    else if (mode == 2) MOE_AL(2);
+    else MOE_AL(0);
+#undef MOE_AL
 #undef MOE_NT
 #undef MOE
+#undef MOE_ARGS
   } else {
     if (tile_rows != 64) return MS_BAD_ARG;
     const dim3 grid(max_tiles, (N + 63) / 64);
     if (grid.y > 65535) return MS_BAD_ARG;
-    if (gated) moe_gemm_f32_kernel<true><<<grid, 256, 0, st>>>((const float*)a, lda, (const float*)w1, (const float*)w2, (float*)out, order, tile_expert, tile_start, tile_count, pair_weight, top, N, K, act);
-    else moe_gemm_f32_kernel<false><<<grid, 256, 0, st>>>((const float*)a, lda, (const float*)w1, nullptr, (float*)out, order, tile_expert, tile_start, tile_count, pair_weight, top, N, K, act);
+#define MOE_F32(G) moe_gemm_f32_kernel<G><<<grid, 256, 0, st>>>((const float*)a, lda, (const float*)w1, (const float*)w2, (float*)out, order, tile_expert, tile_start, tile_count, pair_weight, top, N, K, act)
+    if (mode == 1) MOE_F32(1);
+    else if (mode == 2) MOE_F32(2);
+    else MOE_F32(0);
+#undef MOE_F32
   }
   return launch_status();
 }
 
 // ---------------------------------------------------------------------------------------------
-// stream[t][n] += sum over j < top of y[t * top + j][n], in ascending j.
-__global__ void moe_combine_kernel(float* __restrict__ stream, const float* __restrict__ y, int top, int N) {
+// stream[t][n] += sum over j < top of y[t * top + j][n], in ascending j. With ids: a choice whose id is `real` or more is
+// an identity expert, and its term is weights[t * top + j] * x[t][n] (y holds nothing for it).
+template <typename TX>
+__global__ void moe_combine_kernel(float* __restrict__ stream, const float* __restrict__ y, int top, int N,
+                                   const int* __restrict__ ids, const float* __restrict__ weights, const TX* __restrict__ x,
+                                   int ldx, int real) {
   const int n = blockIdx.x * blockDim.x + threadIdx.x;
   if (n >= N) return;
   const size_t t = blockIdx.y;
   float acc = 0.f;
-  for (int j = 0; j < top; ++j) acc += y[(t * top + j) * N + n];
+  for (int j = 0; j < top; ++j) {
+    if (ids != nullptr && ids[t * top + j] >= real) acc += weights[t * top + j] * to_f32(x[t * ldx + n]);
+    else acc += y[(t * top + j) * N + n];
+  }
   stream[t * N + n] += acc;
 }
 
-extern "C" int ms_moe_combine(float* stream, const float* y, int T, int top, int N, hipStream_t st) {
+extern "C" int ms_moe_combine(float* stream, const float* y, int T, int top, int N, const int* ids, const float* weights,
+                              const void* x, int x_is_bf16, int ldx, int real, hipStream_t st) {
   if (T <= 0 || N <= 0) return MS_OK;
-  if (stream == nullptr || y == nullptr || top < 1 || T > 65535) return MS_BAD_ARG;
-  moe_combine_kernel<<<dim3((N + 255) / 256, T), 256, 0, st>>>(stream, y, top, N);
+  if (stream == nullptr || y == nullptr || top < 1 || T > 65535 || (ids != nullptr && (weights == nullptr || x == nullptr || ldx < N)))
+    return MS_BAD_ARG;
+  const dim3 grid((N + 255) / 256, T);
+  if (x_is_bf16) moe_combine_kernel<bf16><<<grid, 256, 0, st>>>(stream, y, top, N, ids, weights, (const bf16*)x, ldx, real);
+  else moe_combine_kernel<float><<<grid, 256, 0, st>>>(stream, y, top, N, ids, weights, (const float*)x, ldx, real);
   return launch_status();
 }

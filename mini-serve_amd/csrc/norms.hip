@@ -71,14 +71,14 @@ extern "C" int ms_layernorm(const float* x, const void* w, const void* b, int w_
 
 // ---------------------------------------------------------------------------------------------
 // y[t, g * group + e] = x[t, g * group + e] * rsqrt(mean over the group of x^2 + eps) * w[g * group + e]
-//                       * sigmoid(gate[t * gate_stride + g * group + e])
+//                       * sigmoid(gate[t * gate_stride + g * group + e])     (gate_act = 1: SiLU instead of the sigmoid)
 // w == nullptr: no weight; gate == nullptr: no gate. One wave per (token, group) when the group is at
 // most 256 wide (four groups per block), else one block per (token, group).
 template <typename TW, typename TO>
 __global__ __launch_bounds__(256) void group_rmsnorm_gate_kernel(const float* __restrict__ x, const TW* __restrict__ w,
                                                                  const float* __restrict__ gate, int gate_stride,
                                                                  TO* __restrict__ y, int groups, int group, float eps,
-                                                                 int per_wave) {
+                                                                 int per_wave, int gate_act) {
   __shared__ float red[256 / WAVE];
   const int t = blockIdx.x;
   const int width = groups * group;
@@ -104,20 +104,24 @@ __global__ __launch_bounds__(256) void group_rmsnorm_gate_kernel(const float* __
     const int c = g * group + e;
     float o = xr[e] * rstd;
     if (w != nullptr) o *= to_f32(w[c]);
-    if (gate != nullptr) o *= 1.f / (1.f + expf(-gate[(size_t)t * gate_stride + c]));
+    if (gate != nullptr) {
+      const float z = gate[(size_t)t * gate_stride + c];
+      o *= (gate_act ? z : 1.f) / (1.f + expf(-z));  // sigmoid(z), or z sigmoid(z)
+    }
     y[(size_t)t * width + c] = from_f32<TO>(o);
   }
 }
 
 extern "C" int ms_group_rmsnorm_gate(const float* x, const void* w, int w_is_bf16, const float* gate, int gate_stride,
-                                     void* y, int y_is_bf16, int tokens, int groups, int group, float eps, hipStream_t st) {
+                                     void* y, int y_is_bf16, int tokens, int groups, int group, float eps, int gate_act,
+                                     hipStream_t st) {
   if (tokens <= 0) return MS_OK;
-  if (groups <= 0 || group <= 0 || tokens > 65535 * 32 || !(eps >= 0.f) || (gate != nullptr && gate_stride < groups * group))
+  if ((gate_act != 0 && gate_act != 1) || groups <= 0 || group <= 0 || tokens > 65535 * 32 || !(eps >= 0.f) || (gate != nullptr && gate_stride < groups * group))
     return MS_BAD_ARG;
   const int per_wave = group <= 256;
   const dim3 grid(tokens, per_wave ? (groups + 3) / 4 : groups);
   if (grid.y > 65535) return MS_UNSUPPORTED;
-#define GN(TW, TO) group_rmsnorm_gate_kernel<TW, TO><<<grid, 256, 0, st>>>(x, (const TW*)w, gate, gate_stride, (TO*)y, groups, group, eps, per_wave)
+#define GN(TW, TO) group_rmsnorm_gate_kernel<TW, TO><<<grid, 256, 0, st>>>(x, (const TW*)w, gate, gate_stride, (TO*)y, groups, group, eps, per_wave, gate_act)
   if (w_is_bf16) { if (y_is_bf16) GN(bf16, bf16); else GN(bf16, float); }
   else { if (y_is_bf16) GN(float, bf16); else GN(float, float); }
 #undef GN
@@ -247,12 +251,14 @@ extern "C" int ms_scale(float* x, long long n, float s, hipStream_t st) {
 //         the angle whose cosine and sine are rope[t][j] and rope[t][rot/2 + j];
 //   q goes to q_out [tokens, Hq * D]; k and v go to the cache page of the token's slot (keys
 //   [pages, Hkv, page_size, D], values transposed within the page, [pages, Hkv, Dv, page_size]).
-// slots == nullptr: only the queries. One block per token.
+// slots == nullptr: only the queries. One block per token. bias (optional, the row's columns) is added to the projection
+// before anything else; the values are the Hkv * Dv columns from v_col on (behind the keys, or the key columns themselves:
+// values that are the keys as projected, before norm and rotation).
 template <typename T, typename TW>
 __global__ __launch_bounds__(256) void qkv_norm_rope_store_kernel(
     const float* __restrict__ qkv, int ld, T* __restrict__ q_out, const int* __restrict__ slots, const TW* __restrict__ qw,
-    const TW* __restrict__ kw, float eps, const float* __restrict__ rope, int rot, int pairing, T* __restrict__ kc,
-    T* __restrict__ vc, int Hq, int Hkv, int D, int Dv, int page_size) {
+    const TW* __restrict__ kw, const TW* __restrict__ bias, int v_col, float eps, const float* __restrict__ rope, int rot,
+    int pairing, T* __restrict__ kc, T* __restrict__ vc, int Hq, int Hkv, int D, int Dv, int page_size) {
   __shared__ float red[256 / WAVE];
   const int t = blockIdx.x;
   const float* row = qkv + (size_t)t * ld;
@@ -261,23 +267,28 @@ __global__ __launch_bounds__(256) void qkv_norm_rope_store_kernel(
   const float* cs = rot > 0 ? rope + (size_t)t * rot : nullptr;
   const int s = slots ? slots[t] : 0;
   for (int part = 0; part < (slots ? 2 : 1); ++part) {
-    const float* src = row + (part ? nq : 0);
+    const int c0 = part ? nq : 0;  // the part's first column: the bias has the row's columns
+    const float* src = row + c0;
+    const TW* b = bias ? bias + c0 : nullptr;
     const int n = part ? nk : nq;
     const TW* w = part ? kw : qw;
     float rstd = 1.f;
     if (w != nullptr) {
       float ss = 0.f;
-      for (int e = threadIdx.x; e < n; e += 256) ss += src[e] * src[e];
+      for (int e = threadIdx.x; e < n; e += 256) {
+        const float x = src[e] + (b ? to_f32(b[e]) : 0.f);
+        ss += x * x;
+      }
       rstd = 1.f / sqrtf(block_sum<256>(ss, red) / (float)n + eps);
     }
     for (int e = threadIdx.x; e < n; e += 256) {
       const int h = e / D, d = e % D;
-      float v = src[e] * rstd * (w ? to_f32(w[e]) : 1.f);
+      float v = (src[e] + (b ? to_f32(b[e]) : 0.f)) * rstd * (w ? to_f32(w[e]) : 1.f);
       if (d < rot) {
         const bool first = pairing == MS_ROPE_ADJACENT ? (d & 1) == 0 : d < half;
         const int j = pairing == MS_ROPE_ADJACENT ? d / 2 : (d < half ? d : d - half);
         const int pe = e - d + (pairing == MS_ROPE_ADJACENT ? (d ^ 1) : (d < half ? d + half : d - half));
-        const float p = src[pe] * rstd * (w ? to_f32(w[pe]) : 1.f);
+        const float p = (src[pe] + (b ? to_f32(b[pe]) : 0.f)) * rstd * (w ? to_f32(w[pe]) : 1.f);
         v = first ? v * cs[j] - p * cs[half + j] : v * cs[j] + p * cs[half + j];
       }
       if (part == 0) q_out[(size_t)t * nq + e] = from_f32<T>(v);
@@ -285,25 +296,26 @@ __global__ __launch_bounds__(256) void qkv_norm_rope_store_kernel(
     }
   }
   if (slots) {
-    const float* src = row + nq + nk;
+    const float* src = row + v_col;
     for (int e = threadIdx.x; e < nv; e += 256) {
       const int h = e / Dv, d = e % Dv;
-      vc[(((size_t)(s / page_size) * Hkv + h) * Dv + d) * page_size + (s % page_size)] = from_f32<T>(src[e]);
+      const float v = src[e] + (bias ? to_f32(bias[v_col + e]) : 0.f);
+      vc[(((size_t)(s / page_size) * Hkv + h) * Dv + d) * page_size + (s % page_size)] = from_f32<T>(v);
     }
   }
 }
 
 extern "C" int ms_qkv_norm_rope_store(const float* qkv, int ld, void* q_out, int is_bf16, const int* slots, const void* qw,
-                                      const void* kw, int w_is_bf16, float eps, const float* rope, int rot, int pairing,
-                                      void* kc, void* vc, int tokens, int Hq, int Hkv, int D, int Dv, int page_size,
-                                      hipStream_t st) {
+                                      const void* kw, const void* bias, int v_col, int w_is_bf16, float eps, const float* rope,
+                                      int rot, int pairing, void* kc, void* vc, int tokens, int Hq, int Hkv, int D, int Dv,
+                                      int page_size, hipStream_t st) {
   if (tokens <= 0) return MS_OK;
   if (Hq <= 0 || Hkv <= 0 || D <= 0 || Dv <= 0 || page_size <= 0 || rot < 0 || rot > D || rot % 2 || (rot > 0 && rope == nullptr) ||
-      ld < Hq * D + (slots ? Hkv * (D + Dv) : 0) || (slots != nullptr && (kc == nullptr || vc == nullptr)) ||
+      ld < Hq * D + (slots ? Hkv * D : 0) || (slots != nullptr && (kc == nullptr || vc == nullptr || v_col < 0 || v_col + Hkv * Dv > ld)) ||
       (qw == nullptr) != (kw == nullptr) || !(eps >= 0.f))
     return MS_BAD_ARG;
   if (pairing != MS_ROPE_HALVES && pairing != MS_ROPE_ADJACENT) return MS_UNSUPPORTED;
-#define QK(T, TW) qkv_norm_rope_store_kernel<T, TW><<<tokens, 256, 0, st>>>(qkv, ld, (T*)q_out, slots, (const TW*)qw, (const TW*)kw, eps, rope, rot, pairing, (T*)kc, (T*)vc, Hq, Hkv, D, Dv, page_size)
+#define QK(T, TW) qkv_norm_rope_store_kernel<T, TW><<<tokens, 256, 0, st>>>(qkv, ld, (T*)q_out, slots, (const TW*)qw, (const TW*)kw, (const TW*)bias, v_col, eps, rope, rot, pairing, (T*)kc, (T*)vc, Hq, Hkv, D, Dv, page_size)
   if (is_bf16) { if (w_is_bf16) QK(bf16, bf16); else QK(bf16, float); }
   else { if (w_is_bf16) QK(float, bf16); else QK(float, float); }
 #undef QK

@@ -7,6 +7,9 @@
 //       m_t = max(f_t + m_(t-1), i_t) (m starts at 0) that keeps the exponentials in range:
 //       a_t = exp(f_t + m_(t-1) - m_t), b_t = exp(i_t - m_t); a vector n_t = a_t n_(t-1) + b_t k_t beside S;
 //       o_t = S_t^T q_t / (max(|n_t . q_t|, exp(-m_t)) + 1e-6).
+//   MS_REC_WKV: a decay per key channel and token, w_t [D] (row t of the float32 matrix `w`, columns h D ..), and a bonus
+//       u [H, D] that only the current token gets: o_t = (S_(t-1) + diag(u) k_t v_t^T)^T q_t, and only then
+//       S_t = diag(w_t) S_(t-1) + k_t v_t^T.
 // q, k, v (and the gates' inputs) are columns of one float32 matrix x [tokens, ld] (the layer's projections);
 // an activation (none or SiLU) is applied to q, k and v on the way in, q is then scaled by q_scale. Everything
 // is float32. The state lives in S [slots, H, D, E] (and n [slots, H, D], m [slots, H]); a row whose
@@ -23,6 +26,7 @@
 
 #define MS_REC_DECAY 0
 #define MS_REC_EXP_GATES 1
+#define MS_REC_WKV 2
 
 struct RecurrenceArgs {
   const float* x;
@@ -40,6 +44,9 @@ struct RecurrenceArgs {
   const int* starts;
   const int* state_slots;
   float* out;
+  const float* w;  // MS_REC_WKV: the decays [tokens, ld_w], head h's D channels from column h D on
+  int ld_w;
+  const float* u;  // MS_REC_WKV: the bonus [H, D]
 };
 
 __device__ __forceinline__ float rec_act(float v, int act) { return act ? v / (1.f + expf(-v)) : v; }
@@ -51,7 +58,7 @@ __device__ __forceinline__ float log_sigmoid(float z) { return fminf(z, 0.f) - l
 
 template <int PM>
 __global__ __launch_bounds__(256) void gated_recurrence_kernel(RecurrenceArgs a, int EP, int EB) {
-  __shared__ float qs[2][256], ks[2][256];
+  __shared__ float qs[2][256], ks[2][256], ws[2][256], us[256];
   __shared__ float red[256];
   __shared__ float wred[2][4];
   const int b = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
@@ -64,7 +71,8 @@ __global__ __launch_bounds__(256) void gated_recurrence_kernel(RecurrenceArgs a,
   const bool fresh = a.starts[b] == 0;
   const size_t slot = (size_t)a.state_slots[b];
   float* Sg = a.S + (slot * a.H + h) * (size_t)D * E;
-  const bool gates = a.mode == MS_REC_EXP_GATES;
+  const bool gates = a.mode == MS_REC_EXP_GATES, wkv = a.mode == MS_REC_WKV;
+  if (wkv && tid < D) us[tid] = a.u[h * D + tid];  // read behind the first token's barrier
   float S[PM];
 #pragma unroll
   for (int i = 0; i < PM; ++i) {
@@ -76,7 +84,7 @@ __global__ __launch_bounds__(256) void gated_recurrence_kernel(RecurrenceArgs a,
     if (tid < D) nv = a.n[(slot * a.H + h) * D + tid];
     m = a.m[slot * a.H + h];
   }
-  const float decay = gates ? 0.f : a.decay[h];
+  const float decay = (gates || wkv) ? 0.f : a.decay[h];
   const float bi = gates ? rec_bias(a.i_bias, a.bias_is_bf16, h) : 0.f;
   const float bf = gates ? rec_bias(a.f_bias, a.bias_is_bf16, h) : 0.f;
   for (int t = t0; t < t1; ++t) {
@@ -97,6 +105,7 @@ __global__ __launch_bounds__(256) void gated_recurrence_kernel(RecurrenceArgs a,
       kd = rec_act(xr[a.k_off + h * D + tid], a.act);
       qs[buf][tid] = qd;
       ks[buf][tid] = kd;
+      if (wkv) ws[buf][tid] = a.w[(size_t)t * a.ld_w + h * D + tid];
     }
     if (gates) {
       nv = fs * nv + is * kd;  // threads beyond D carry zeros
@@ -110,8 +119,14 @@ __global__ __launch_bounds__(256) void gated_recurrence_kernel(RecurrenceArgs a,
     for (int i = 0; i < PM; ++i) {
       const int d = s + i * NS;
       if (i < per && d < D) {
-        S[i] = fs * S[i] + is * ks[buf][d] * v;
-        acc += S[i] * qs[buf][d];
+        if (wkv) {
+          const float kv = ks[buf][d] * v;
+          acc += (S[i] + us[d] * kv) * qs[buf][d];
+          S[i] = ws[buf][d] * S[i] + kv;
+        } else {
+          S[i] = fs * S[i] + is * ks[buf][d] * v;
+          acc += S[i] * qs[buf][d];
+        }
       }
     }
     if (NS > 1) {
@@ -145,7 +160,8 @@ __global__ __launch_bounds__(256) void gated_recurrence_kernel(RecurrenceArgs a,
 extern "C" int ms_gated_recurrence(const float* x, int ld, int q_off, int k_off, int v_off, int i_off, int f_off, int H, int D,
                                    int E, int act, int mode, float q_scale, float cap, const float* decay, const void* i_bias,
                                    const void* f_bias, int bias_is_bf16, float* S, float* n, float* m, const int* row_start,
-                                   const int* starts, const int* state_slots, float* out, int rows, hipStream_t st) {
+                                   const int* starts, const int* state_slots, float* out, int rows, const float* w, int ld_w,
+                                   const float* u, hipStream_t st) {
   if (rows <= 0) return MS_OK;
   if (H <= 0 || D <= 0 || E <= 0 || x == nullptr || S == nullptr || out == nullptr || row_start == nullptr || starts == nullptr ||
       state_slots == nullptr || (act != 0 && act != 1) || q_off < 0 || k_off < 0 || v_off < 0 || q_off + H * D > ld ||
@@ -155,6 +171,8 @@ extern "C" int ms_gated_recurrence(const float* x, int ld, int q_off, int k_off,
     if (decay == nullptr) return MS_BAD_ARG;
   } else if (mode == MS_REC_EXP_GATES) {
     if (n == nullptr || m == nullptr || !(cap > 0.f) || i_off < 0 || f_off < 0 || i_off + H > ld || f_off + H > ld) return MS_BAD_ARG;
+  } else if (mode == MS_REC_WKV) {
+    if (w == nullptr || u == nullptr || ld_w < H * D) return MS_BAD_ARG;
   } else {
     return MS_BAD_ARG;
   }
@@ -163,7 +181,7 @@ extern "C" int ms_gated_recurrence(const float* x, int ld, int q_off, int k_off,
   const int EB = E < 32 ? E : 32, EP = 32;
   const int per = (D + 256 / EP - 1) / (256 / EP);
   RecurrenceArgs a{x, ld, q_off, k_off, v_off, i_off, f_off, H, D, E, act, mode, q_scale, cap, decay, i_bias, f_bias, bias_is_bf16,
-                   S, n, m, row_start, starts, state_slots, out};
+                   S, n, m, row_start, starts, state_slots, out, w, ld_w, u};
   const dim3 grid(rows, H, (E + EB - 1) / EB);
   if (per <= 4) gated_recurrence_kernel<4><<<grid, 256, 0, st>>>(a, EP, EB);
   else if (per <= 16) gated_recurrence_kernel<16><<<grid, 256, 0, st>>>(a, EP, EB);

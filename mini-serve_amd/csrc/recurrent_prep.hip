@@ -1,0 +1,112 @@
+// What recurrent mixers do to their projections before the recurrence runs, all in float32:
+//   * a rotation of the query and key heads of a float32 projection, in place, with a scale on the way;
+//   * the blends of a token's input with the previous token's, one per projection, and the carry of the last input;
+//   * a decay per channel and token out of a small two-step projection.
+#include "common.h"
+
+// ---------------------------------------------------------------------------------------------
+// x[t, col + h D + d] for h < H, d < D, in place: the first `rot` elements of each head are turned in pairs (j, j + rot/2)
+// (or (2j, 2j + 1)) by the angles of rope[t] (cosines, then sines), then every element of the head is multiplied by
+// `scale`. A thread owns a pair, or one element behind the rotated part: nothing is read by one thread and written by
+// another. One block per token.
+__global__ __launch_bounds__(256) void rotate_columns_kernel(float* __restrict__ x, int ld, int col, int H, int D,
+                                                             const float* __restrict__ rope, int rot, int pairing, float scale) {
+  const int t = blockIdx.x;
+  float* row = x + (size_t)t * ld + col;
+  const int half = rot / 2;
+  const int per = D - half;  // items of a head: rot / 2 pairs and D - rot single elements
+  const float* cs = rot > 0 ? rope + (size_t)t * rot : nullptr;
+  for (int item = threadIdx.x; item < H * per; item += 256) {
+    const int h = item / per, i = item % per;
+    float* hd = row + h * D;
+    if (i < half) {
+      const int a = pairing == MS_ROPE_ADJACENT ? 2 * i : i;
+      const int b = pairing == MS_ROPE_ADJACENT ? 2 * i + 1 : i + half;
+      const float u = hd[a], v = hd[b];
+      const float c = cs[i], s = cs[half + i];
+      hd[a] = (u * c - v * s) * scale;
+      hd[b] = (v * c + u * s) * scale;
+    } else {
+      hd[i + half] *= scale;  // element rot + (i - rot / 2)
+    }
+  }
+}
+
+extern "C" int ms_rotate_columns(float* x, int ld, int col, int tokens, int H, int D, const float* rope, int rot, int pairing,
+                                 float scale, hipStream_t st) {
+  if (tokens <= 0) return MS_OK;
+  if (x == nullptr || H <= 0 || D <= 0 || col < 0 || col + H * D > ld || rot < 0 || rot > D || rot % 2 || (rot > 0 && rope == nullptr))
+    return MS_BAD_ARG;
+  if (pairing != MS_ROPE_HALVES && pairing != MS_ROPE_ADJACENT) return MS_UNSUPPORTED;
+  rotate_columns_kernel<<<tokens, 256, 0, st>>>(x, ld, col, H, D, rope, rot, pairing, scale);
+  return launch_status();
+}
+
+// ---------------------------------------------------------------------------------------------
+// out[s][t][c] = h[t][c] + (prev[t][c] - h[t][c]) * mu[s][c] for s < n: prev is the row before t in the step when t is not
+// the first token of its request's rows, else the request's carried row carry[slot] (zeros when the request starts in this
+// step). Float32 arithmetic, rounded once. The thread that reads carry[slot][c] for a request's first token is the one that
+// then writes the request's last row of this step there: one reader and one writer per element, the same thread.
+template <typename T>
+__global__ __launch_bounds__(256) void token_shift_mix_kernel(const T* __restrict__ h, const T* __restrict__ mu, T* __restrict__ out,
+                                                              float* __restrict__ carry, const int* __restrict__ token_row,
+                                                              const int* __restrict__ row_start, const int* __restrict__ starts,
+                                                              const int* __restrict__ state_slots, int tokens, int W, int n) {
+  const int t = blockIdx.x;
+  const int row = token_row[t];
+  const int t0 = row_start[row], t1 = row_start[row + 1];
+  const bool first = t == t0;
+  const bool fresh = starts[row] == 0;
+  float* cr = carry + (size_t)state_slots[row] * W;
+  const T* hr = h + (size_t)t * W;
+  const T* pr = first ? nullptr : h + (size_t)(t - 1) * W;
+  const T* last = h + (size_t)(t1 - 1) * W;
+  for (int c = threadIdx.x; c < W; c += 256) {
+    const float x = to_f32(hr[c]);
+    const float p = first ? (fresh ? 0.f : cr[c]) : to_f32(pr[c]);
+    const float back = p - x;
+    for (int s = 0; s < n; ++s) out[((size_t)s * tokens + t) * W + c] = from_f32<T>(x + back * to_f32(mu[(size_t)s * W + c]));
+    if (first) cr[c] = to_f32(last[c]);
+  }
+}
+
+extern "C" int ms_token_shift_mix(const void* h, const void* mu, void* out, int is_bf16, float* carry, const int* token_row,
+                                  const int* row_start, const int* starts, const int* state_slots, int tokens, int W, int n,
+                                  hipStream_t st) {
+  if (tokens <= 0) return MS_OK;
+  if (h == nullptr || mu == nullptr || out == nullptr || carry == nullptr || token_row == nullptr || row_start == nullptr ||
+      starts == nullptr || state_slots == nullptr || W <= 0 || n <= 0)
+    return MS_BAD_ARG;
+  if (is_bf16) token_shift_mix_kernel<bf16><<<tokens, 256, 0, st>>>((const bf16*)h, (const bf16*)mu, (bf16*)out, carry, token_row, row_start, starts, state_slots, tokens, W, n);
+  else token_shift_mix_kernel<float><<<tokens, 256, 0, st>>>((const float*)h, (const float*)mu, (float*)out, carry, token_row, row_start, starts, state_slots, tokens, W, n);
+  return launch_status();
+}
+
+// ---------------------------------------------------------------------------------------------
+// out[t][c] = exp(-exp(sum_r w2t[r][c] tanh(a[t][col + r]) + w0[c])), c < C, r < R: the decay of channel c at token t.
+// a: float32 [tokens, lda] (the first step's projection); w2t: the second step's weight transposed, [R, C]; w0 [C].
+// Float32 throughout, the sum in ascending r. One block per token; tanh(a[t]) goes through LDS.
+#define DECAY_MAX_RANK 1024
+template <typename TW>
+__global__ __launch_bounds__(256) void channel_decay_kernel(const float* __restrict__ a, int lda, int col, const TW* __restrict__ w2t,
+                                                            const TW* __restrict__ w0, float* __restrict__ out, int C, int R) {
+  __shared__ float th[DECAY_MAX_RANK];
+  const int t = blockIdx.x;
+  for (int r = threadIdx.x; r < R; r += 256) th[r] = tanhf(a[(size_t)t * lda + col + r]);
+  __syncthreads();
+  for (int c = threadIdx.x; c < C; c += 256) {
+    float z = 0.f;
+    for (int r = 0; r < R; ++r) z = fmaf(to_f32(w2t[(size_t)r * C + c]), th[r], z);
+    out[(size_t)t * C + c] = expf(-expf(z + to_f32(w0[c])));
+  }
+}
+
+extern "C" int ms_channel_decay(const float* a, int lda, int col, const void* w2t, const void* w0, int w_is_bf16, float* out,
+                                int tokens, int C, int R, hipStream_t st) {
+  if (tokens <= 0) return MS_OK;
+  if (a == nullptr || w2t == nullptr || w0 == nullptr || out == nullptr || C <= 0 || R <= 0 || col < 0 || col + R > lda) return MS_BAD_ARG;
+  if (R > DECAY_MAX_RANK) return MS_UNSUPPORTED;
+  if (w_is_bf16) channel_decay_kernel<bf16><<<tokens, 256, 0, st>>>(a, lda, col, (const bf16*)w2t, (const bf16*)w0, out, C, R);
+  else channel_decay_kernel<float><<<tokens, 256, 0, st>>>(a, lda, col, (const float*)w2t, (const float*)w0, out, C, R);
+  return launch_status();
+}

@@ -269,7 +269,7 @@ __global__ void activate_kernel(const float* __restrict__ x, T* __restrict__ out
 
 extern "C" int ms_activate(const float* x, void* out, int out_is_bf16, long long n, int act, hipStream_t st) {
   if (n <= 0) return MS_OK;
-  if (act < 0 || act >= MS_ACT_COUNT) return MS_BAD_ARG;
+  if (!ms_act_ungated_ok(act)) return MS_BAD_ARG;
   const unsigned blocks = (unsigned)((n + 255) / 256);
   if (out_is_bf16) activate_kernel<bf16><<<blocks, 256, 0, st>>>(x, (bf16*)out, (size_t)n, act);
   else activate_kernel<float><<<blocks, 256, 0, st>>>(x, (float*)out, (size_t)n, act);

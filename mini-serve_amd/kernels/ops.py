@@ -27,16 +27,19 @@ _SIGNATURES = {
     "ms_act_mul": [_c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_void],
     "ms_act_mul_parts": [_c_void, _c_int, _c_ll, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_void],
     "ms_layernorm": [_c_void, _c_void, _c_void, _c_int, _c_void, _c_int, _c_void, _c_int, _c_int, _c_float, _c_void],
-    "ms_group_rmsnorm_gate": [_c_void, _c_void, _c_int, _c_void, _c_int, _c_void, _c_int, _c_int, _c_int, _c_int, _c_float, _c_void],
+    "ms_group_rmsnorm_gate": [_c_void, _c_void, _c_int, _c_void, _c_int, _c_void, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_void],
     "ms_normed_mean_add": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _c_void],
     "ms_normed_add_pending": [_c_void, _c_void, _c_void, _c_int, _c_ll, _c_void, _c_int, _c_int, _c_int, _c_float, _c_void, _c_int,
                               _c_void],
     "ms_scale": [_c_void, _c_ll, _c_float, _c_void],
-    "ms_qkv_norm_rope_store": [_c_void, _c_int, _c_void, _c_int, _c_void, _c_void, _c_void, _c_int, _c_float, _c_void, _c_int, _c_int,
-                               _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
+    "ms_qkv_norm_rope_store": [_c_void, _c_int, _c_void, _c_int, _c_void, _c_void, _c_void, _c_void, _c_int, _c_int, _c_float, _c_void,
+                               _c_int, _c_int, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
     "ms_gated_recurrence": [_c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float,
                             _c_float, _c_void, _c_void, _c_void, _c_int, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void,
-                            _c_int, _c_void],
+                            _c_int, _c_void, _c_int, _c_void, _c_void],
+    "ms_rotate_columns": [_c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void, _c_int, _c_int, _c_float, _c_void],
+    "ms_token_shift_mix": [_c_void, _c_void, _c_void, _c_int, _c_void, _c_void, _c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_void],
+    "ms_channel_decay": [_c_void, _c_int, _c_int, _c_void, _c_void, _c_int, _c_void, _c_int, _c_int, _c_int, _c_void],
     "ms_gated_recurrence_chunked": [_c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
                                     _c_float, _c_float, _c_void, _c_void, _c_void, _c_int, _c_void, _c_void, _c_void, _c_void, _c_void,
                                     _c_void, _c_void, _c_int, _c_int, _c_void, _c_void, _c_void, _c_void],
@@ -100,10 +103,11 @@ _SIGNATURES = {
                               _c_int, _c_void, _c_int, _c_float, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
                               _c_void],
     "ms_moe_route": [_c_void, _c_int, _c_int, _c_ll, _c_void, _c_int, _c_int, _c_int, _c_int, _c_void, _c_void, _c_void],
+    "ms_moe_route_scored": [_c_void, _c_int, _c_int, _c_ll, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void, _c_void, _c_void],
     "ms_moe_plan": [_c_void, _c_int, _c_int, _c_int, _c_int, _c_void, _c_void, _c_void, _c_void, _c_void],
     "ms_moe_gemm": [_c_void, _c_int, _c_void, _c_void, _c_void, _c_int, _c_int, _c_void, _c_void, _c_void, _c_void, _c_void,
                     _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
-    "ms_moe_combine": [_c_void, _c_void, _c_int, _c_int, _c_int, _c_void],
+    "ms_moe_combine": [_c_void, _c_void, _c_int, _c_int, _c_int, _c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_void],
     "ms_measure_read": [_c_void, _c_ll, _c_int, _c_void, _c_void],
     "ms_measure_copy": [_c_void, _c_void, _c_ll, _c_int, _c_void],
 }
@@ -294,15 +298,18 @@ def interleave_gate_up(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
 # silu(x) = x sigmoid(x); gelu_tanh(x) = x / 2 (1 + tanh(sqrt(2 / pi) (x + 0.044715 x^3))).
 # swiglu_clamped(gate, up) = g sigmoid(1.702 g) (u + 1) with g = min(gate, limit), u = clamp(up, -limit, limit): not of
 # the form act(gate) * up, it takes ``limit`` along and runs in the activation kernels (no matrix kernel's epilogue knows it).
-ACTIVATIONS = {"silu": 0, "gelu_tanh": 1, "swiglu_clamped": 2}
+ACTIVATIONS = {"silu": 0, "gelu_tanh": 1, "swiglu_clamped": 2, "relu_squared": 3}
+ACTIVATIONS_UNGATED_ONLY = {"relu_squared"}  # no kernel finishes act(gate) * up with these
 ACTIVATIONS_WITH_LIMIT = {"swiglu_clamped"}
 
 
-def _activation(name: str, limit: float | None = None) -> int:
+def _activation(name: str, limit: float | None = None, gated: bool = True) -> int:
     try:
         act = ACTIVATIONS[name]
     except KeyError:
         raise NotImplementedError(f"activation {name!r}: the kernels know {sorted(ACTIVATIONS)}") from None
+    if gated and name in ACTIVATIONS_UNGATED_ONLY:
+        raise NotImplementedError(f"activation {name!r} has no gated form act(gate) * up here")
     if name in ACTIVATIONS_WITH_LIMIT and not (limit is not None and limit > 0):
         raise ValueError(f"activation {name!r} needs a positive limit, got {limit!r}")
     return act
@@ -383,7 +390,7 @@ MAX_STEP_TOKENS = 65535  # rows one launch of the matrix and elementwise kernels
 
 
 def linear(x: torch.Tensor, weight: torch.Tensor, out_dtype=None, accumulate_into: torch.Tensor | None = None,
-           defer: bool = False):
+           defer: bool = False, out: torch.Tensor | None = None):
     """``x [M, K] @ weight [N, K]^T``. Either returns a new ``[M, N]`` tensor of ``out_dtype``, or adds
     the product into the float32 tensor ``accumulate_into`` (the residual stream) and returns None.
     The weight's dtype picks the arithmetic: float32 weights run the true 32-bit kernel (``x`` is
@@ -391,38 +398,54 @@ def linear(x: torch.Tensor, weight: torch.Tensor, out_dtype=None, accumulate_int
 
     ``defer=True`` allows the result to come back as a ``SplitSum`` (partial sums that the consuming
     kernel adds up) where the small-M kernel produced it in that form; with ``accumulate_into`` the
-    returned ``SplitSum`` is what still has to be added to that tensor."""
+    returned ``SplitSum`` is what still has to be added to that tensor.
+
+    ``out``: a float32 ``[M, N]`` view of a wider matrix (unit column stride, rows a multiple of four floats apart and
+    the first element 16-byte aligned) that receives the product; it is returned. Several products then share one
+    matrix whose columns a later kernel reads side by side."""
     _dev(x, "x", (F32, BF16), 2)
     _dev(weight, "weight", (F32, BF16), 2)
     m, k = x.shape
     n = weight.shape[0]
     if weight.shape[1] != k:
         raise ValueError(f"linear: x is [{m}, {k}], weight is {tuple(weight.shape)}")
+    ldc = n
+    if out is not None:
+        if accumulate_into is not None or defer:
+            raise ValueError("linear: out= goes with neither accumulate_into nor defer")
+        if not (isinstance(out, torch.Tensor) and out.is_cuda and out.dtype == F32 and out.dim() == 2 and tuple(out.shape) == (m, n)
+                and out.stride(1) == 1 and out.stride(0) >= n and out.stride(0) % 4 == 0 and out.data_ptr() % 16 == 0):
+            raise ValueError(f"linear: out must be a float32 [{m}, {n}] view with unit column stride, rows a multiple of 4 floats "
+                             "apart and a 16-byte aligned start")
+        ldc = out.stride(0)
     if accumulate_into is not None:
         _dev(accumulate_into, "accumulate_into", F32, 2)
         if tuple(accumulate_into.shape) != (m, n):
             raise ValueError(f"linear: accumulator is {tuple(accumulate_into.shape)}, expected {(m, n)}")
-    elif out_dtype not in (F32, BF16):
+    elif out is None and out_dtype not in (F32, BF16):
         raise TypeError(f"unsupported output dtype {out_dtype}")
     lib = library()
     if weight.dtype == BF16 and m <= SMALL_M:
         xa = cast(x, BF16)
         splits = lib.ms_gemm_bf16_small_splits(m, n, k)
-        if splits == 1 and accumulate_into is None and out_dtype == F32:
-            out = torch.empty((m, n), dtype=F32, device=x.device)  # the single partial sum is the result
-            _check(lib.ms_gemm_bf16_small(xa.data_ptr(), weight.data_ptr(), out.data_ptr(), None, 1, 0, m, n, k, k, n,
+        if splits == 1 and accumulate_into is None and out is None and out_dtype == F32:
+            res = torch.empty((m, n), dtype=F32, device=x.device)  # the single partial sum is the result
+            _check(lib.ms_gemm_bf16_small(xa.data_ptr(), weight.data_ptr(), res.data_ptr(), None, 1, 0, m, n, k, k, n,
                                           _stream()), "gemm_bf16_small")
-            return out
+            return res
         parts = torch.empty((splits, m, n), dtype=F32, device=x.device)
         if defer:
             _check(lib.ms_gemm_bf16_small(xa.data_ptr(), weight.data_ptr(), parts.data_ptr(), None, 1, 0, m, n, k, k, n,
                                           _stream()), "gemm_bf16_small")
             return SplitSum(parts)
-        out = accumulate_into if accumulate_into is not None else torch.empty((m, n), dtype=out_dtype, device=x.device)
-        mode = 2 if accumulate_into is not None else (1 if out.dtype == F32 else 0)
-        _check(lib.ms_gemm_bf16_small(xa.data_ptr(), weight.data_ptr(), parts.data_ptr(), out.data_ptr(), mode, 1, m, n, k,
-                                      k, n, _stream()), "gemm_bf16_small")
-        return None if accumulate_into is not None else out
+        if out is not None:
+            res = out
+        else:
+            res = accumulate_into if accumulate_into is not None else torch.empty((m, n), dtype=out_dtype, device=x.device)
+        mode = 2 if accumulate_into is not None else (1 if res.dtype == F32 else 0)
+        _check(lib.ms_gemm_bf16_small(xa.data_ptr(), weight.data_ptr(), parts.data_ptr(), res.data_ptr(), mode, 1, m, n, k,
+                                      k, ldc, _stream()), "gemm_bf16_small")
+        return None if accumulate_into is not None else res
     if weight.dtype == BF16 and defer:
         splits = lib.ms_gemm_bf16_tile_splits(m, n, k)
         if splits > 1:  # few output tiles: split K over the grid and leave the sum to the consumer
@@ -431,16 +454,19 @@ def linear(x: torch.Tensor, weight: torch.Tensor, out_dtype=None, accumulate_int
             _check(lib.ms_gemm_bf16(xa.data_ptr(), weight.data_ptr(), parts.data_ptr(), 1, m, n, k, k, n, splits, _stream()),
                    "gemm_bf16")
             return SplitSum(parts)
-    out = accumulate_into if accumulate_into is not None else torch.empty((m, n), dtype=out_dtype, device=x.device)
+    if out is not None:
+        res = out
+    else:
+        res = accumulate_into if accumulate_into is not None else torch.empty((m, n), dtype=out_dtype, device=x.device)
     if weight.dtype == F32:
         xa = cast(x, F32)
-        mode = 1 if accumulate_into is not None else (0 if out.dtype == F32 else 2)
-        _check(lib.ms_gemm_f32(xa.data_ptr(), weight.data_ptr(), out.data_ptr(), mode, m, n, k, k, n, _stream()), "gemm_f32")
+        mode = 1 if accumulate_into is not None else (0 if res.dtype == F32 else 2)
+        _check(lib.ms_gemm_f32(xa.data_ptr(), weight.data_ptr(), res.data_ptr(), mode, m, n, k, k, ldc, _stream()), "gemm_f32")
     else:
         xa = cast(x, BF16)
-        mode = 2 if accumulate_into is not None else (1 if out.dtype == F32 else 0)
-        _check(lib.ms_gemm_bf16(xa.data_ptr(), weight.data_ptr(), out.data_ptr(), mode, m, n, k, k, n, 1, _stream()), "gemm_bf16")
-    return None if accumulate_into is not None else out
+        mode = 2 if accumulate_into is not None else (1 if res.dtype == F32 else 0)
+        _check(lib.ms_gemm_bf16(xa.data_ptr(), weight.data_ptr(), res.data_ptr(), mode, m, n, k, k, ldc, 1, _stream()), "gemm_bf16")
+    return None if accumulate_into is not None else res
 
 
 def tile_shape(m: int, n: int, k: int, splits: int = 1, gated: bool = False) -> tuple[int, int] | None:
@@ -470,10 +496,16 @@ MOE_SMALL_TILE_PAIRS = 16  # (token, expert) pairs per expert, on average, up to
 MOE_LARGE_TILE_PAIRS = 128  # ... and from which it runs 128-pair tiles (widths that are multiples of 64)
 
 
-def moe_route(logits, bias: torch.Tensor | None, top: int):
-    """Per row of the float32 router logits ``[T, E]`` (plus ``bias [E]``): the ``top`` experts with the largest values,
-    largest first (ties: the lower index), as int32 ``[T, top]``, and the softmax over those values alone, float32
-    ``[T, top]``. The logits may be a ``SplitSum``: the kernel adds the partial sums itself."""
+def moe_route(logits, bias: torch.Tensor | None, top: int, scoring: str = "chosen_softmax", groups: int = 1, keep: int = 1):
+    """Per row of the float32 router logits ``[T, E]``: the ``top`` chosen outputs, best first (ties: the lower index), as
+    int32 ``[T, top]``, and their weights, float32 ``[T, top]``. The logits may be a ``SplitSum``: the kernel adds the
+    partial sums itself.
+
+    ``scoring="chosen_softmax"``: the choice goes by ``logits + bias``, the weights are the softmax over the chosen values
+    alone. ``scoring="softmax"``: ``s = softmax(logits)`` over all ``E`` outputs; the choice goes by ``s + bias`` (a
+    correction that only the choice sees), the weights are the chosen outputs' ``s`` as they stand; with ``groups > 1``
+    the outputs form that many equal groups of neighbours, a group's score is the largest ``s + bias`` in it, and only
+    outputs of the ``keep`` best groups can be chosen."""
     if isinstance(logits, SplitSum):
         parts, splits, stride = logits.parts, logits.splits, logits.stride
         _dev(parts, "logits", F32, 3)
@@ -486,38 +518,55 @@ def moe_route(logits, bias: torch.Tensor | None, top: int):
         raise ValueError(f"top {top} of {e} experts")
     if e > MOE_MAX_EXPERTS or top > MOE_MAX_TOP:
         raise ValueError(f"{e} experts / top {top}: the routing kernel takes up to {MOE_MAX_EXPERTS} experts and {MOE_MAX_TOP} choices")
+    if scoring not in ("chosen_softmax", "softmax"):
+        raise NotImplementedError(f"router scoring {scoring!r}: 'chosen_softmax' or 'softmax'")
     if bias is not None:
         _dev(bias, "bias", (F32, BF16), 1)
         if bias.shape[0] != e:
             raise ValueError(f"the router's bias has {bias.shape[0]} elements for {e} experts")
     ids = torch.empty((t, top), dtype=I32, device=parts.device)
     weights = torch.empty((t, top), dtype=F32, device=parts.device)
+    if scoring == "softmax":
+        if groups < 1 or e % groups or not 1 <= keep <= groups:
+            raise ValueError(f"{e} router outputs in {groups} groups of which {keep} are kept")
+        if top > (e // groups) * keep:
+            raise ValueError(f"top {top} of the {(e // groups) * keep} outputs in the kept groups")
+        _check(library().ms_moe_route_scored(parts.data_ptr(), e, splits, stride, _ptr(bias), int(bias is not None and bias.dtype == BF16),
+                                             t, e, top, int(groups), int(keep), ids.data_ptr(), weights.data_ptr(), _stream()),
+               "moe_route_scored")
+        return ids, weights
+    if groups != 1:
+        raise NotImplementedError("groups of experts go with scoring='softmax'")
     _check(library().ms_moe_route(parts.data_ptr(), e, splits, stride, _ptr(bias), int(bias is not None and bias.dtype == BF16), t, e,
                                   top, ids.data_ptr(), weights.data_ptr(), _stream()), "moe_route")
     return ids, weights
 
 
-def moe_experts(x: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, gate: torch.Tensor, up: torch.Tensor,
+def moe_experts(x: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, gate: torch.Tensor | None, up: torch.Tensor,
                 down: torch.Tensor, activation: str, stream: torch.Tensor) -> None:
-    """``stream[t] += sum_j weights[t, j] * down[e] (act(gate[e] x[t]) * (up[e] x[t]))`` with ``e = ids[t, j]``, the sum in
-    ascending ``j``. ``x [T, W]`` in the compute dtype, ``gate`` / ``up`` ``[E, F, W]`` and ``down [E, W, F]`` in the same,
-    ``stream`` float32 ``[T, W]``. The step's (token, expert) pairs are sorted by expert on the device and every expert's
-    run is multiplied in tiles (bfloat16: on the matrix cores; float32: fused multiply-adds in ascending k); the launches
-    cover the most tiles the step can have, so nothing is read back and a captured step replays."""
-    act = _activation(activation)
-    if act >= 2:
+    """``stream[t] += sum_j weights[t, j] * expert_e(x[t])`` with ``e = ids[t, j]``, the sum in ascending ``j``. A gated
+    expert is ``down[e] (act(gate[e] x) * (up[e] x))``; with ``gate=None`` it is ``down[e] act(up[e] x)``. An id of
+    ``E`` (the number of experts that have weights) or more names an identity expert: its term is ``weights[t, j] * x[t]``.
+    ``x [T, W]`` in the compute dtype, ``gate`` / ``up`` ``[E, F, W]`` and ``down [E, W, F]`` in the same, ``stream`` float32
+    ``[T, W]``. The step's (token, expert) pairs are sorted by expert on the device and every expert's run is multiplied
+    in tiles (bfloat16: on the matrix cores; float32: fused multiply-adds in ascending k); the launches cover the most
+    tiles the step can have, so nothing is read back and a captured step replays."""
+    gated = gate is not None
+    act = _activation(activation, gated=gated)
+    if act == ACTIVATIONS["swiglu_clamped"]:
         raise NotImplementedError(f"activation {activation!r} is not of the form act(gate) * up")
     _dev(x, "x", (F32, BF16), 2)
     for w, nm in ((gate, "gate"), (up, "up"), (down, "down")):
-        _dev(w, nm, x.dtype, 3)
+        if w is not None:
+            _dev(w, nm, x.dtype, 3)
     _dev(ids, "ids", I32, 2)
     _dev(weights, "weights", F32, 2)
     _dev(stream, "stream", F32, 2)
     t, width = x.shape
-    e, f = gate.shape[0], gate.shape[1]
+    e, f = up.shape[0], up.shape[1]
     top = ids.shape[1]
-    if gate.shape != (e, f, width) or up.shape != (e, f, width) or down.shape != (e, width, f):
-        raise ValueError(f"expert weights {tuple(gate.shape)} / {tuple(up.shape)} / {tuple(down.shape)} do not fit x {tuple(x.shape)}")
+    if (gated and gate.shape != (e, f, width)) or up.shape != (e, f, width) or down.shape != (e, width, f):
+        raise ValueError(f"expert weights {tuple(up.shape)} / {tuple(down.shape)} do not fit x {tuple(x.shape)}")
     if ids.shape[0] != t or tuple(weights.shape) != tuple(ids.shape) or tuple(stream.shape) != (t, width):
         raise ValueError("ids, weights and stream must have one row per row of x")
     if e > MOE_MAX_EXPERTS:
@@ -530,7 +579,7 @@ def moe_experts(x: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, gate:
     bf = x.dtype == BF16
     tile_rows = 16 if bf and pairs <= MOE_SMALL_TILE_PAIRS * e else 64
     if bf and pairs >= MOE_LARGE_TILE_PAIRS * e and width % 64 == 0 and f % 64 == 0 and not any(
-            t.data_ptr() % 16 for t in (x, gate, up, down)):
+            w.data_ptr() % 16 for w in (x, gate, up, down) if w is not None):
         tile_rows = 128  # both products then run tiles of 128 pairs staged through LDS
     max_tiles = -(-pairs // tile_rows) + min(e, pairs)
     dev = x.device
@@ -541,12 +590,13 @@ def moe_experts(x: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, gate:
                            tiles[2].data_ptr(), _stream()), "moe_plan")
     plan = (order.data_ptr(), tiles[0].data_ptr(), tiles[1].data_ptr(), tiles[2].data_ptr())
     h = torch.empty((pairs, f), dtype=x.dtype, device=dev)
-    _check(lib.ms_moe_gemm(x.data_ptr(), width, gate.data_ptr(), up.data_ptr(), h.data_ptr(), int(bf), 1, *plan, None, max_tiles, top,
-                           f, width, tile_rows, act, _stream()), "moe_gemm")
+    _check(lib.ms_moe_gemm(x.data_ptr(), width, (gate if gated else up).data_ptr(), up.data_ptr() if gated else None, h.data_ptr(), int(bf),
+                           1 if gated else 2, *plan, None, max_tiles, top, f, width, tile_rows, act, _stream()), "moe_gemm")
     y = torch.empty((pairs, width), dtype=F32, device=dev)
     _check(lib.ms_moe_gemm(h.data_ptr(), f, down.data_ptr(), None, y.data_ptr(), int(bf), 0, *plan, weights.data_ptr(), max_tiles, top,
                            width, f, tile_rows, act, _stream()), "moe_gemm")
-    _check(lib.ms_moe_combine(stream.data_ptr(), y.data_ptr(), t, top, width, _stream()), "moe_combine")
+    _check(lib.ms_moe_combine(stream.data_ptr(), y.data_ptr(), t, top, width, ids.data_ptr(), weights.data_ptr(), x.data_ptr(), int(bf),
+                              width, e, _stream()), "moe_combine")
 
 
 # ------------------------------------------------------------------------------------- attention
@@ -1099,11 +1149,16 @@ def layernorm(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, 
     return out
 
 
+GATE_ACTIVATIONS = {"sigmoid": 0, "silu": 1}  # what a gate goes through before it multiplies a normed output
+
+
 def group_rmsnorm_gate(x: torch.Tensor, group: int, weight: torch.Tensor | None, gate: torch.Tensor | None, eps: float,
-                       out_dtype) -> torch.Tensor:
-    """``x / rms(group of x) * weight * sigmoid(gate)`` for float32 ``x [T, N]`` cut into groups of ``group``
+                       out_dtype, gate_activation: str = "sigmoid") -> torch.Tensor:
+    """``x / rms(group of x) * weight * act(gate)`` for float32 ``x [T, N]`` cut into groups of ``group``
     consecutive elements (``group == N``: one norm over the row). ``weight [N]`` and ``gate`` (float32 ``[T, N]``,
-    may be a column slice of a wider matrix) are optional."""
+    may be a column slice of a wider matrix) are optional; ``gate_activation``: ``"sigmoid"`` or ``"silu"``."""
+    if gate_activation not in GATE_ACTIVATIONS:
+        raise NotImplementedError(f"gate activation {gate_activation!r}: the kernel knows {sorted(GATE_ACTIVATIONS)}")
     _dev(x, "x", F32, 2)
     t, n = x.shape
     if group < 1 or n % group:
@@ -1122,7 +1177,7 @@ def group_rmsnorm_gate(x: torch.Tensor, group: int, weight: torch.Tensor | None,
     out = torch.empty((t, n), dtype=out_dtype, device=x.device)
     _check(library().ms_group_rmsnorm_gate(x.data_ptr(), _ptr(weight), int(weight is not None and weight.dtype == BF16), _ptr(gate),
                                            gate_stride, out.data_ptr(), int(out_dtype == BF16), t, n // group, group, float(eps),
-                                           _stream()), "group_rmsnorm_gate")
+                                           GATE_ACTIVATIONS[gate_activation], _stream()), "group_rmsnorm_gate")
     return out
 
 
@@ -1183,30 +1238,48 @@ def scale_(x: torch.Tensor, factor: float) -> torch.Tensor:
 
 
 def qkv_norm_rope_store(qkv, slots, q_weight, k_weight, eps, rope, k_cache, v_cache, num_heads, num_kv_heads, head_dim,
-                        value_dim, out_dtype, pairing: str = "halves") -> torch.Tensor:
-    """From float32 ``qkv [T, Hq D + Hkv D + Hkv Dv]``: RMS norm of the whole query part and of the whole key
+                        value_dim, out_dtype, pairing: str = "halves", bias: torch.Tensor | None = None,
+                        values_are_keys: bool = False, extra_columns: int = 0) -> torch.Tensor:
+    """From float32 ``qkv [T, Hq D + Hkv D + Hkv Dv]`` (and ``extra_columns`` more behind them that are not read here): RMS norm of the whole query part and of the whole key
     part of a token (weights ``[Hq D]`` and ``[Hkv D]``; None: no norm), rotation of the first ``rope.shape[1]``
     elements of each query and key head, in pairs as ``pairing`` names them, by the angles of ``rope`` (a
     ``rope_table`` of these tokens; None: no rotation), keys and values stored into the cache pages at ``slots``
-    (skipped when ``slots`` is None). Returns the finished queries ``[T, Hq D]`` in ``out_dtype``."""
+    (skipped when ``slots`` is None). Returns the finished queries ``[T, Hq D]`` in ``out_dtype``.
+
+    ``bias`` (one element per column that is read) is added to the projection first. ``values_are_keys``: the matrix has
+    no value columns; a token's values are its keys as projected, bias included, before norm and rotation
+    (``value_dim == head_dim``)."""
     _dev(qkv, "qkv", F32, 2)
     t = qkv.shape[0]
-    width = num_heads * head_dim + num_kv_heads * (head_dim + value_dim)
-    if qkv.shape[1] != width:
-        raise ValueError(f"qkv has width {qkv.shape[1]}, expected {width}")
+    nq, nk = num_heads * head_dim, num_kv_heads * head_dim
+    if values_are_keys:
+        if value_dim != head_dim:
+            raise ValueError(f"values that are the keys have the keys' size {head_dim}, not {value_dim}")
+        width, v_col = nq + nk, nq
+    else:
+        width, v_col = nq + nk + num_kv_heads * value_dim, nq + nk
+    if extra_columns < 0 or qkv.shape[1] != width + extra_columns:
+        raise ValueError(f"qkv has width {qkv.shape[1]}, expected {width + extra_columns}")
     if out_dtype not in (F32, BF16):
         raise TypeError(f"unsupported output dtype {out_dtype}")
-    w_bf16 = 0
+    w_bf16 = None
     if (q_weight is None) != (k_weight is None):
         raise ValueError("the query and the key norm come together or not at all")
     if q_weight is not None:
-        for w, nm, n in ((q_weight, "q_norm", num_heads * head_dim), (k_weight, "k_norm", num_kv_heads * head_dim)):
+        for w, nm, n in ((q_weight, "q_norm", nq), (k_weight, "k_norm", nk)):
             _dev(w, nm, (F32, BF16), 1)
             if w.shape[0] != n:
                 raise ValueError(f"{nm} weight has {w.shape[0]} elements, expected {n}")
         if q_weight.dtype != k_weight.dtype:
             raise TypeError("q_norm and k_norm weights differ in dtype")
         w_bf16 = int(q_weight.dtype == BF16)
+    if bias is not None:
+        _dev(bias, "bias", (F32, BF16), 1)
+        if bias.shape[0] != width:
+            raise ValueError(f"the bias has {bias.shape[0]} elements for {width} columns")
+        if w_bf16 is not None and int(bias.dtype == BF16) != w_bf16:
+            raise TypeError("the bias and the norm weights differ in dtype")
+        w_bf16 = int(bias.dtype == BF16)
     page_size = 1
     if slots is not None:
         _dev(slots, "slots", I32, 1)
@@ -1219,10 +1292,10 @@ def qkv_norm_rope_store(qkv, slots, q_weight, k_weight, eps, rope, k_cache, v_ca
         rot_dim = rope.shape[1]
         if rope.shape[0] != t or rot_dim % 2 or rot_dim > head_dim or rot_dim < 2:
             raise ValueError(f"rotation table is {tuple(rope.shape)}; {t} tokens and an even width up to {head_dim} are needed")
-    q_out = torch.empty((t, num_heads * head_dim), dtype=out_dtype, device=qkv.device)
+    q_out = torch.empty((t, nq), dtype=out_dtype, device=qkv.device)
     _check(library().ms_qkv_norm_rope_store(
-        qkv.data_ptr(), qkv.shape[1], q_out.data_ptr(), int(out_dtype == BF16), _ptr(slots), _ptr(q_weight), _ptr(k_weight), w_bf16,
-        float(eps), _ptr(rope), int(rot_dim), pair, _ptr(k_cache) if slots is not None else None,
+        qkv.data_ptr(), qkv.shape[1], q_out.data_ptr(), int(out_dtype == BF16), _ptr(slots), _ptr(q_weight), _ptr(k_weight), _ptr(bias),
+        v_col, int(w_bf16 or 0), float(eps), _ptr(rope), int(rot_dim), pair, _ptr(k_cache) if slots is not None else None,
         _ptr(v_cache) if slots is not None else None, t, num_heads, num_kv_heads, head_dim, int(value_dim), page_size, _stream()),
         "qkv_norm_rope_store")
     return q_out
@@ -1474,7 +1547,7 @@ def head_linear(x: torch.Tensor, weights: torch.Tensor, out: torch.Tensor, out_c
 
 DECODE_GENERIC_WAVES = 16  # waves that share a (token, head) in the float32 attention of single-token rows (8 or 16)
 
-RECURRENCE_MODES = {"decay": 0, "exp_gates": 1}
+RECURRENCE_MODES = {"decay": 0, "exp_gates": 1, "wkv": 2}
 RECURRENCE_MAX_DIM = 256
 RECURRENCE_CHUNKED_FROM = 16  # tokens of the longest row from which a step runs the chunked kernels
 
@@ -1482,7 +1555,7 @@ RECURRENCE_CHUNKED_FROM = 16  # tokens of the longest row from which a step runs
 def gated_recurrence(x: torch.Tensor, columns: dict, heads: int, dim: int, value_dim: int, batch, state: dict, *,
                      mode: str, activation: str | None = None, q_scale: float = 1.0, decay: torch.Tensor | None = None,
                      cap: float = 0.0, i_bias: torch.Tensor | None = None, f_bias: torch.Tensor | None = None,
-                     chunks: bool = True) -> torch.Tensor:
+                     chunks: bool = True, channel_decay: torch.Tensor | None = None, bonus: torch.Tensor | None = None) -> torch.Tensor:
     """A linear recurrence over a matrix state per (request, head): ``S_t = a_t S_(t-1) + b_t k_t v_t^T``,
     ``o_t = S_t^T q_t``, for the step's rows (``batch.row_start``, ``batch.starts``, ``batch.state_slots``), in float32.
 
@@ -1491,6 +1564,9 @@ def gated_recurrence(x: torch.Tensor, columns: dict, heads: int, dim: int, value
     each). ``activation`` (None or ``"silu"``) is applied to q, k and v; q is then scaled by ``q_scale``.
     ``mode="decay"``: ``a = decay[head]``, ``b = 1``. ``mode="exp_gates"``: capped exponential gates with a running
     maximum and a normaliser (the kernel's source states the formulas); ``state`` then also holds ``n`` and ``m``.
+    ``mode="wkv"``: a decay per key channel and token, ``channel_decay`` (float32 ``[T, heads * dim]``), and a ``bonus``
+    (float32 ``[heads, dim]``) for the current token alone: ``o_t = (S_(t-1) + diag(bonus) k_t v_t^T)^T q_t``, then
+    ``S_t = diag(channel_decay_t) S_(t-1) + k_t v_t^T``.
     ``state["S"]``: float32 ``[slots, heads, dim, value_dim]``; rows with ``starts == 0`` begin from zero.
     Returns float32 ``[T, heads * value_dim]``.
 
@@ -1527,6 +1603,13 @@ def gated_recurrence(x: torch.Tensor, columns: dict, heads: int, dim: int, value
                     raise ValueError(f"{nm} has {b_.shape[0]} elements for {heads} heads")
         if i_bias is not None and f_bias is not None and i_bias.dtype != f_bias.dtype:
             raise TypeError("the gates' biases differ in dtype")
+    elif mode == "wkv":
+        _dev(channel_decay, "channel_decay", F32, 2)
+        _dev(bonus, "bonus", F32, 2)
+        if tuple(channel_decay.shape) != (t, heads * dim) or tuple(bonus.shape) != (heads, dim):
+            raise ValueError(f"channel_decay {tuple(channel_decay.shape)} / bonus {tuple(bonus.shape)} do not fit {t} tokens of "
+                             f"{heads} heads of {dim}")
+        chunks = False  # the chunked kernels know one decay per head and token
     else:
         _dev(decay, "decay", F32, 1)
         if decay.shape[0] != heads:
@@ -1565,7 +1648,72 @@ def gated_recurrence(x: torch.Tensor, columns: dict, heads: int, dim: int, value
         x.data_ptr(), ld, columns["q"], columns["k"], columns["v"], columns.get("i", 0), columns.get("f", 0), heads, dim, value_dim,
         int(activation == "silu"), RECURRENCE_MODES[mode], float(q_scale), float(cap), _ptr(decay), _ptr(i_bias), _ptr(f_bias),
         int(bias is not None and bias.dtype == BF16), S.data_ptr(), _ptr(n), _ptr(m), batch.row_start.data_ptr(),
-        batch.starts.data_ptr(), batch.state_slots.data_ptr(), out.data_ptr(), rows, _stream()), "gated_recurrence")
+        batch.starts.data_ptr(), batch.state_slots.data_ptr(), out.data_ptr(), rows, _ptr(channel_decay), heads * dim, _ptr(bonus),
+        _stream()), "gated_recurrence")
+    return out
+
+
+def rotate_columns_(x: torch.Tensor, col: int, heads: int, dim: int, rope: torch.Tensor | None, pairing: str = "halves",
+                    scale: float = 1.0) -> torch.Tensor:
+    """In place on the float32 ``x [T, ld]``: the ``heads`` heads of ``dim`` elements from column ``col`` on have their
+    first ``rope.shape[1]`` elements turned by the angles of ``rope`` (a ``rope_table`` of these tokens; None: no
+    rotation), and every element of them is then multiplied by ``scale``."""
+    _dev(x, "x", F32, 2)
+    t = x.shape[0]
+    rot = 0
+    if rope is not None:
+        _dev(rope, "rope", F32, 2)
+        rot = rope.shape[1]
+        if rope.shape[0] != t or rot % 2 or rot > dim:
+            raise ValueError(f"rotation table is {tuple(rope.shape)}; {t} tokens and an even width up to {dim} are needed")
+    if col < 0 or col + heads * dim > x.shape[1]:
+        raise ValueError(f"columns {col} .. {col + heads * dim} lie outside the matrix of width {x.shape[1]}")
+    if rot == 0 and scale == 1.0:
+        return x
+    _check(library().ms_rotate_columns(x.data_ptr(), x.shape[1], int(col), t, heads, dim, _ptr(rope), rot, _pairing(pairing), float(scale),
+                                       _stream()), "rotate_columns")
+    return x
+
+
+def token_shift_mix(h: torch.Tensor, mu: torch.Tensor, carry: torch.Tensor, batch) -> torch.Tensor:
+    """``out[s, t] = h[t] + (h[t - 1] - h[t]) * mu[s]`` for every blend ``s``: ``h [T, W]`` and ``mu [n, W]`` in one dtype,
+    the result ``[n, T, W]`` in the same (float32 arithmetic, rounded once). ``h[t - 1]`` of a row's first token is the row
+    its request carried in ``carry [slots, W]`` (float32; zeros where the request starts in this step), and the row's last
+    token of this step is carried from here on."""
+    _dev(h, "h", (F32, BF16), 2)
+    _dev(mu, "mu", h.dtype, 2)
+    _dev(carry, "carry", F32, 2)
+    t, w = h.shape
+    if mu.shape[1] != w or carry.shape[1] != w:
+        raise ValueError(f"mu {tuple(mu.shape)} / carry {tuple(carry.shape)} do not fit rows of {w}")
+    for v_, nm in ((batch.token_row, "token_row"), (batch.row_start, "row_start"), (batch.starts, "starts"), (batch.state_slots, "state_slots")):
+        _dev(v_, nm, I32, 1)
+    if batch.num_tokens != t or batch.token_row.shape[0] != t:
+        raise ValueError("one row of h per token of the step is needed")
+    out = torch.empty((mu.shape[0], t, w), dtype=h.dtype, device=h.device)
+    _check(library().ms_token_shift_mix(h.data_ptr(), mu.data_ptr(), out.data_ptr(), int(h.dtype == BF16), carry.data_ptr(),
+                                        batch.token_row.data_ptr(), batch.row_start.data_ptr(), batch.starts.data_ptr(),
+                                        batch.state_slots.data_ptr(), t, w, mu.shape[0], _stream()), "token_shift_mix")
+    return out
+
+
+CHANNEL_DECAY_MAX_RANK = 1024  # DECAY_MAX_RANK in csrc/recurrent_prep.hip
+
+
+def channel_decay(a: torch.Tensor, col: int, w2t: torch.Tensor, w0: torch.Tensor) -> torch.Tensor:
+    """``exp(-exp(tanh(a[:, col : col + R]) @ w2t + w0))``: float32 ``[T, C]`` from the float32 ``a [T, >= col + R]``,
+    ``w2t [R, C]`` and ``w0 [C]`` (one dtype), float32 arithmetic, the sum in ascending ``r``."""
+    _dev(a, "a", F32, 2)
+    _dev(w2t, "w2t", (F32, BF16), 2)
+    _dev(w0, "w0", w2t.dtype, 1)
+    r, c = w2t.shape
+    if col < 0 or col + r > a.shape[1] or w0.shape[0] != c:
+        raise ValueError(f"columns {col} .. {col + r} of a matrix of width {a.shape[1]}, w0 of {w0.shape[0]} for {c} channels")
+    if r > CHANNEL_DECAY_MAX_RANK:
+        raise ValueError(f"a first step of {r} outputs: the kernel takes up to {CHANNEL_DECAY_MAX_RANK}")
+    out = torch.empty((a.shape[0], c), dtype=F32, device=a.device)
+    _check(library().ms_channel_decay(a.data_ptr(), a.shape[1], int(col), w2t.data_ptr(), w0.data_ptr(), int(w2t.dtype == BF16),
+                                      out.data_ptr(), a.shape[0], c, r, _stream()), "channel_decay")
     return out
 
 # ------------------------------------------------------------------------------------- sampling

@@ -19,7 +19,11 @@ positions; the cache keeps their pages); ``value_dim`` (size of a value head, de
 ``qk_norm="projection"`` (the RMS norm runs over a token's whole query projection and over its whole key
 projection, before they are split into heads, with weights of those sizes; default ``"head"``);
 ``exact_weights`` (the softmax weights meet the values in float32: no rounding of them to bfloat16 for the
-matrix cores); ``names`` (the tensors' names behind the prefix, by ``q k v o q_norm k_norm sink blend``).
+matrix cores); ``names`` (the tensors' names behind the prefix, by ``q k v o q_norm k_norm sink blend q_bias k_bias
+v_bias gate``); ``bias`` (the projections have biases, added before anything else); ``values_are_keys`` (there is no
+value projection: a token's values are its keys as projected, bias included, before norm and rotation);
+``head_gate`` (a tensor ``[heads, hidden]``: head ``h``'s output is multiplied by ``sigmoid(gate x)_h`` before the output
+projection). The last three run the path with one norm over the projection.
 
 And four more, which run the path whose every step between projection and attention is a parameter of one kernel
 (``ops.head_prepare_store``): ``qk_norm="head_rotated"`` (the norm per head sits behind the rotation instead of before
@@ -46,7 +50,8 @@ def _names(spec: PartSpec) -> dict[str, str]:
     p = spec.get("prefix", "")
     given = spec.get("names") or {}
     default = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight",
-               "q_norm": "q_norm.weight", "k_norm": "k_norm.weight", "sink": "sinks", "blend": "value_blend"}
+               "q_norm": "q_norm.weight", "k_norm": "k_norm.weight", "sink": "sinks", "blend": "value_blend",
+               "q_bias": "q_proj.bias", "k_bias": "k_proj.bias", "v_bias": "v_proj.bias", "gate": "gate.weight"}
     return {k: p + given.get(k, d) for k, d in default.items()}
 
 
@@ -71,6 +76,11 @@ class GQAttention(Mixer):
         self.sinks = bool(spec.get("sinks", False))
         self.value_blend = spec.get("value_blend")
         self.blend_key = ("value_blend", spec.get("blend_group", "values"))
+        self.bias = bool(spec.get("bias", False))
+        self.values_are_keys = bool(spec.get("values_are_keys", False))
+        self.head_gate = bool(spec.get("head_gate", False))
+        if self.values_are_keys and self.value_dim != self.head_dim:
+            raise ValueError(f"values that are the keys have the keys' size {self.head_dim}, not {self.value_dim}")
         if self.qk_norm not in ("head", "projection", "head_rotated"):
             raise ValueError(f"qk_norm {self.qk_norm!r}: 'head', 'projection' or 'head_rotated'")
         if self.value_blend not in (None, "first", "blend"):
@@ -80,10 +90,14 @@ class GQAttention(Mixer):
                          or (self.qk_norm_eps is not None and not self.qk_norm_weights))
         if self.prepared and (self.qk_norm == "projection" or self.keep_first):
             raise NotImplementedError("sinks, blended values and a norm behind the rotation go with a norm per head and no kept first keys")
+        extras = self.bias or self.values_are_keys or self.head_gate
+        if extras and (self.prepared or (self.qk_norm == "head" and self.qk_norm_eps is not None)):
+            raise NotImplementedError("biases, values that are the keys and a gate per head go with one norm over the projection or none")
         if self.keep_first < 0 or self.window < 0:
             raise ValueError("window and keep_first must not be negative")
         # The path with one norm over the projection, values of their own size, kept first keys or unrounded weights.
-        self.wide = not self.prepared and ((self.qk_norm == "projection" and self.qk_norm_eps is not None) or self.value_dim != self.head_dim)
+        self.wide = not self.prepared and ((self.qk_norm == "projection" and self.qk_norm_eps is not None)
+                                           or self.value_dim != self.head_dim or extras)
         if self.wide and self.qk_norm == "head" and self.qk_norm_eps is not None:
             raise NotImplementedError("a norm per head together with values of another size than the keys is not supported")
         if self.heads % self.kv_heads:
@@ -103,8 +117,9 @@ class GQAttention(Mixer):
                 "with up to 16 query heads per KV head", stacklevel=2)
         pos = spec.get("position") or PartSpec("none")
         self.position = part_class("position", pos)(pos, rt)
-        self.qkv = self.o = self.q_norm = self.k_norm = self.sink = None
+        self.qkv = self.o = self.q_norm = self.k_norm = self.sink = self.qkv_bias = None
         self.blend = 0.0
+        self.gate_col = 0
 
     @classmethod
     def tensors(cls, spec: PartSpec) -> dict[str, TensorSpec]:
@@ -112,12 +127,21 @@ class GQAttention(Mixer):
         h, d = int(spec["hidden_size"]), int(spec["head_dim"])
         dv = int(spec.get("value_dim") or d)
         hq, hkv = int(spec["num_heads"]), int(spec["num_kv_heads"])
+        own_values = not spec.get("values_are_keys", False)
         out = {
             n["q"]: TensorSpec((hq * d, h)),
             n["k"]: TensorSpec((hkv * d, h)),
-            n["v"]: TensorSpec((hkv * dv, h)),
             n["o"]: TensorSpec((h, hq * dv)),
         }
+        if own_values:
+            out[n["v"]] = TensorSpec((hkv * dv, h))
+        if spec.get("bias", False):
+            out[n["q_bias"]] = TensorSpec((hq * d,), init="uniform")
+            out[n["k_bias"]] = TensorSpec((hkv * d,), init="uniform")
+            if own_values:
+                out[n["v_bias"]] = TensorSpec((hkv * dv,), init="uniform")
+        if spec.get("head_gate", False):
+            out[n["gate"]] = TensorSpec((hq, h))
         if spec.get("qk_norm_eps") is not None and spec.get("qk_norm_weights", True):
             whole = spec.get("qk_norm", "head") == "projection"
             out[n["q_norm"]] = TensorSpec((hq * d if whole else d,), init="ones")
@@ -131,7 +155,16 @@ class GQAttention(Mixer):
 
     def bind(self, tensors) -> None:
         p, n = self.prefix, self.names
-        parts = [tensors[n[k]] for k in ("q", "k", "v")]
+        kinds = ("q", "k") if self.values_are_keys else ("q", "k", "v")
+        parts = [tensors[n[k]] for k in kinds]
+        if self.bias:
+            biases = [tensors[n[k + "_bias"]] for k in kinds]
+            if len({t.dtype for t in biases}) != 1:
+                raise ValueError(f"{p}the projections' biases are stored in different dtypes")
+            self.qkv_bias = torch.cat(biases, dim=0).contiguous()
+        if self.head_gate:
+            self.gate_col = sum(t.shape[0] for t in parts)  # the gate's rows lie behind the projections
+            parts.append(tensors[n["gate"]])
         if len({t.dtype for t in parts}) != 1:
             raise ValueError(f"{p}q/k/v projections are stored in different dtypes")
         self.qkv = torch.cat(parts, dim=0).contiguous()
@@ -159,9 +192,11 @@ class GQAttention(Mixer):
             qkv = ops.linear(x, self.qkv, out_dtype=torch.float32)  # the norms' input is not rounded
             q = ops.qkv_norm_rope_store(qkv, cache.slots if cache.writes else None, self.q_norm, self.k_norm, eps, table,
                                         cache.k, cache.v, self.heads, self.kv_heads, self.head_dim, self.value_dim,
-                                        self.rt.dtype, pairing)
+                                        self.rt.dtype, pairing, self.qkv_bias, self.values_are_keys, self.heads if self.head_gate else 0)
             out = ops.paged_attention(q, cache.k, cache.v, cache.block_table, batch, self.heads, self.kv_heads, self.head_dim,
                                       self.scale, self.window, self.value_dim, self.keep_first, self.exact_weights)
+            if self.head_gate:
+                ops.head_gate_(out, qkv, self.gate_col, self.heads)
             return ops.linear(out, self.o, accumulate_into=residual, defer=True)
         qkv = ops.linear(x, self.qkv, out_dtype=self.rt.dtype, defer=True)
         if not (self.exact_weights or self.keep_first) and ops.decode_attention_fusable(qkv, batch, self.q_norm, self.k_norm, table, cache.k, cache.v,
@@ -214,7 +249,8 @@ class GQAttention(Mixer):
         return ops.linear(out, self.o, accumulate_into=residual, defer=True)
 
     def parameters_bytes(self) -> int:
-        ts = [self.qkv, self.o] + ([self.q_norm, self.k_norm] if self.q_norm is not None else []) + ([self.sink] if self.sink is not None else [])
+        ts = [self.qkv, self.o] + ([self.q_norm, self.k_norm] if self.q_norm is not None else []) + [
+            t for t in (self.sink, self.qkv_bias) if t is not None]
         return sum(t.numel() * t.element_size() for t in ts)
 
     def flops(self, rows) -> int:
@@ -228,5 +264,6 @@ class GQAttention(Mixer):
             if not self.window:
                 pairs += n * cached + n * (n + 1) // 2
         qk, vo = self.heads * self.head_dim, self.heads * self.value_dim
-        linear = 2 * tokens * self.hidden * (qk + self.kv_heads * (self.head_dim + self.value_dim)) + 2 * tokens * vo * self.hidden
+        projected = qk + self.kv_heads * (self.head_dim + (0 if self.values_are_keys else self.value_dim)) + (self.heads if self.head_gate else 0)
+        linear = 2 * tokens * self.hidden * projected + 2 * tokens * vo * self.hidden
         return linear + 2 * pairs * (qk + vo)

@@ -40,15 +40,27 @@ class TensorSpec:
     ``"ones"`` a scale around one (norm weights: all one, or uniform in the range the caller gives),
     ``"uniform"`` U(-std, std), ``"zeros"`` (a bias that starts switched off); integer tables are
     drawn uniformly from ``[0, high)``. ``optional``: a checkpoint may hold the tensor or not; nothing reads it
-    (the loader accepts it, the random-weights mode does not draw it, the part is not handed it)."""
+    (the loader accepts it, the random-weights mode does not draw it, the part is not handed it).
 
-    shape: tuple[int, ...]
+    A dimension of ``None`` is free: the checkpoint's size is taken as it comes and the part reads it off the tensor it
+    is bound to (a size that no configuration key states); the random-weights mode draws ``free`` there."""
+
+    shape: tuple
     kind: str = "float"
     init: str = "normal"
     high: int | None = None
     optional: bool = False
+    free: int | None = None
+
+    def fits(self, shape) -> bool:
+        return len(shape) == len(self.shape) and all(w is None or w == g for w, g in zip(self.shape, shape))
+
+    def drawn_shape(self) -> tuple[int, ...]:
+        return tuple(self.free if d is None else d for d in self.shape)
 
     def __post_init__(self):
+        if any(d is None for d in self.shape) and (self.free is None or self.free < 1):
+            raise ValueError("a tensor with a free dimension needs ``free``: the size the random-weights mode draws")
         if self.kind not in ("float", "int"):
             raise ValueError(f"unknown tensor kind {self.kind!r}")
         if self.kind == "float" and self.init not in ("normal", "ones", "uniform", "zeros"):

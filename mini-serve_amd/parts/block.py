@@ -1,6 +1,6 @@
 """Block arrangements: where the norms and the residual sums sit around a mixer and a
 feed-forward. ``prenorm`` is the reference's (miniserve/model/qwen3.py:212-216):
-``h += mixer(norm(h)); h += feed_forward(norm(h))``. ``parallel`` and ``outnorm`` have no counterpart there."""
+``h += mixer(norm(h)); h += feed_forward(norm(h))``. ``parallel``, ``outnorm`` and ``sandwich`` have no counterpart there."""
 
 from __future__ import annotations
 
@@ -136,3 +136,56 @@ class OutputNormBlock(Block):
 
     def parameters_bytes(self) -> int:
         return self.mixer_norm.parameters_bytes() + (self.ffn_norm.parameters_bytes() if self.ffn_norm is not None else 0)
+
+
+@register("block", "sandwich")
+class SandwichBlock(Block):
+    """``h += out1(mixer(in1(h))); h += out2(feed_forward(in2(h)))``: a norm in front of every sublayer and another
+    behind it. The norms in front are the pre-norm block's (``mixer_norm``, ``ffn_norm``), the ones behind the
+    output-norm block's (``mixer_out_norm``, ``ffn_out_norm``): each sublayer adds into a stream that starts at zero,
+    and the norm behind it folds that stream into the residual stream and leaves it zero again. A layer without a
+    feed-forward has neither ``ffn_norm`` nor ``ffn_out_norm`` (None); ``spare`` then names norm tensors
+    ``{name: width}`` that a checkpoint may still carry for them."""
+
+    NORMS = ("mixer_norm", "mixer_out_norm", "ffn_norm", "ffn_out_norm")
+
+    def __init__(self, spec: PartSpec, rt, mixer, feed_forward):
+        super().__init__(spec, rt, mixer, feed_forward)
+        if (spec.get("ffn_norm") is None) != (spec.get("ffn_out_norm") is None):
+            raise ValueError("the feed-forward's two norms come together or not at all")
+        self.norms = {k: part_class("norm", spec[k])(spec[k], rt) if spec.get(k) is not None else None for k in self.NORMS}
+
+    @classmethod
+    def tensors(cls, spec: PartSpec) -> dict[str, TensorSpec]:
+        out = {}
+        for key in cls.NORMS:
+            s = spec.get(key)
+            if s is not None:
+                out.update(part_class("norm", s).tensors(s))
+        for name, width in (spec.get("spare") or {}).items():
+            out[name] = TensorSpec((int(width),), optional=True)
+        return out
+
+    def bind(self, tensors) -> None:
+        for n in self.norms.values():
+            if n is not None:
+                n.bind(tensors)
+
+    def forward(self, residual, batch, cache, state, pending=None):
+        n = self.norms
+        key = ("outnorm_stream", tuple(residual.shape))  # one zeroed stream per pass, shared with the output-norm blocks
+        own = batch.memo.get(key)
+        if own is None:
+            own = batch.memo[key] = torch.zeros_like(residual)
+        batch.memo.pop(ROUNDED_RESIDUAL, None)  # the norm in front reads the stream itself
+        x = n["mixer_norm"].forward(residual, add=pending)
+        first = self.mixer.forward(x, batch, cache, state, own)
+        n["mixer_out_norm"].add_normed(residual, own, first, clear=True)
+        if n["ffn_norm"] is not None:
+            y = n["ffn_norm"].forward(residual)
+            second = self.feed_forward.forward(y, own)
+            n["ffn_out_norm"].add_normed(residual, own, second, clear=True)
+        return None
+
+    def parameters_bytes(self) -> int:
+        return sum(n.parameters_bytes() for n in self.norms.values() if n is not None)

@@ -16,7 +16,16 @@ runs ``top``: router logits ``router x (+ router_bias)`` in float32, the ``top``
 weights the softmax over the chosen logits alone, the output the weighted sum of the chosen experts' outputs. ``shared``
 (optional) is the ``PartSpec`` of any registered feed-forward that runs for every token and is added. ``names`` maps
 ``router``, ``router_bias``, ``expert`` (a pattern with ``{}`` for the expert's number, behind the prefix) and ``gate`` /
-``up`` / ``down`` (behind the expert's own prefix)."""
+``up`` / ``down`` (behind the expert's own prefix).
+
+Further parameters of ``moe_mlp`` (the defaults give the mixture above): ``gated=False`` (an expert is
+``down(act(up x))``, no ``gate`` tensors; ``activation`` may then be any that has an ungated form, ``relu_squared``
+among them); ``scoring="softmax"`` (the router's softmax runs over all its outputs; the choice goes by the softmax
+value plus ``router_bias``, a correction that only the choice sees; the weights are the chosen outputs' softmax values
+as they stand, not renormalised); ``groups`` / ``keep_groups`` (with that scoring: the router's outputs form ``groups``
+equal groups of neighbours, a group's score is the largest choice score in it, and only outputs of the ``keep_groups``
+best groups can be chosen); ``identity`` (the router has that many outputs more than there are experts with weights; a
+token that chooses one of them gets its own input back, times the weight)."""
 
 from __future__ import annotations
 
@@ -49,8 +58,9 @@ class GatedMLP(FeedForward):
         self.inter = int(spec["intermediate_size"])
         self.activation = spec.get("activation", "silu")
         self.limit = float(spec["limit"]) if spec.get("limit") is not None else None
-        if self.activation not in rt.ops.ACTIVATIONS:
-            raise NotImplementedError(f"activation {self.activation!r} is not supported, expected one of {sorted(rt.ops.ACTIVATIONS)}")
+        if self.activation not in rt.ops.ACTIVATIONS or self.activation in rt.ops.ACTIVATIONS_UNGATED_ONLY:
+            raise NotImplementedError(f"activation {self.activation!r} is not supported, expected one of "
+                                      f"{sorted(set(rt.ops.ACTIVATIONS) - set(rt.ops.ACTIVATIONS_UNGATED_ONLY))}")
         if self.activation in rt.ops.ACTIVATIONS_WITH_LIMIT and not (self.limit is not None and self.limit > 0):
             raise ValueError(f"activation {self.activation!r} needs a positive limit, got {self.limit!r}")
         self.names = _names(spec)
@@ -137,14 +147,30 @@ class MixtureMLP(FeedForward):
         self.top = int(spec["top"])
         self.activation = spec.get("activation", "silu")
         self.router_bias = bool(spec.get("router_bias", False))
-        if not 1 <= self.top <= self.num_experts:
-            raise ValueError(f"top {self.top} of {self.num_experts} experts")
+        self.gated = bool(spec.get("gated", True))
+        self.scoring = spec.get("scoring", "chosen_softmax")
+        self.groups = int(spec.get("groups") or 1)
+        self.keep_groups = int(spec.get("keep_groups") or self.groups)
+        self.identity = int(spec.get("identity") or 0)
+        self.outputs = self.num_experts + self.identity  # what the router tells apart
+        if self.scoring not in ("chosen_softmax", "softmax"):
+            raise ValueError(f"router scoring {self.scoring!r}: 'chosen_softmax' or 'softmax'")
+        if self.identity < 0 or self.num_experts < 1:
+            raise ValueError(f"{self.num_experts} experts and {self.identity} identity experts")
+        if self.groups != 1 and self.scoring != "softmax":
+            raise NotImplementedError("groups of experts go with scoring='softmax'")
+        if self.groups < 1 or self.outputs % self.groups or not 1 <= self.keep_groups <= self.groups:
+            raise ValueError(f"{self.outputs} router outputs in {self.groups} groups of which {self.keep_groups} are kept")
+        if not 1 <= self.top <= (self.outputs // self.groups) * self.keep_groups:
+            raise ValueError(f"top {self.top} of {self.outputs} router outputs in {self.groups} groups of which {self.keep_groups} are kept")
         if rt is not None:
             ops = rt.ops
-            if self.activation not in ops.ACTIVATIONS or self.activation in ops.ACTIVATIONS_WITH_LIMIT:
-                raise NotImplementedError(f"activation {self.activation!r} is not of the form act(gate) * up")
-            if self.num_experts > ops.MOE_MAX_EXPERTS or self.top > ops.MOE_MAX_TOP:
-                raise ValueError(f"{self.num_experts} experts / top {self.top}: the kernels take up to {ops.MOE_MAX_EXPERTS} "
+            if self.activation not in ops.ACTIVATIONS or self.activation in ops.ACTIVATIONS_WITH_LIMIT or (
+                    self.gated and self.activation in ops.ACTIVATIONS_UNGATED_ONLY):
+                raise NotImplementedError(f"activation {self.activation!r} is not of the form "
+                                          f"{'act(gate) * up' if self.gated else 'act(up)'}")
+            if self.outputs > ops.MOE_MAX_EXPERTS or self.top > ops.MOE_MAX_TOP:
+                raise ValueError(f"{self.outputs} experts / top {self.top}: the kernels take up to {ops.MOE_MAX_EXPERTS} "
                                  f"experts and {ops.MOE_MAX_TOP} choices")
         self.names = _moe_names(spec)
         sh = spec.get("shared")
@@ -160,12 +186,15 @@ class MixtureMLP(FeedForward):
     def tensors(cls, spec: PartSpec) -> dict[str, TensorSpec]:
         n, p = _moe_names(spec), spec.get("prefix", "")
         h, i, e = int(spec["hidden_size"]), int(spec["intermediate_size"]), int(spec["num_experts"])
-        out = {p + n["router"]: TensorSpec((e, h))}
+        outputs = e + int(spec.get("identity") or 0)
+        out = {p + n["router"]: TensorSpec((outputs, h))}
         if spec.get("router_bias", False):
-            out[p + n["router_bias"]] = TensorSpec((e,), init="uniform")
+            out[p + n["router_bias"]] = TensorSpec((outputs,), init="uniform")
         for j in range(e):
             en = cls._expert_names(spec, j)
-            out[en["gate"]], out[en["up"]], out[en["down"]] = TensorSpec((i, h)), TensorSpec((i, h)), TensorSpec((h, i))
+            out[en["up"]], out[en["down"]] = TensorSpec((i, h)), TensorSpec((h, i))
+            if spec.get("gated", True):
+                out[en["gate"]] = TensorSpec((i, h))
         sh = spec.get("shared")
         if sh is not None:
             out.update(part_class("feed_forward", sh).tensors(sh))
@@ -175,11 +204,13 @@ class MixtureMLP(FeedForward):
         n, p = self.names, self.prefix
         self.router = tensors[p + n["router"]]
         self.bias = tensors[p + n["router_bias"]] if self.router_bias else None
-        per = [self._expert_names(self.spec, j) for j in range(self.num_experts)]
+        kinds = ("gate", "up", "down") if self.gated else ("up", "down")
+        per = [{k: v for k, v in self._expert_names(self.spec, j).items() if k in kinds} for j in range(self.num_experts)]
         if len({tensors[en[k]].dtype for en in per for k in en}) != 1:
             raise ValueError(f"{p}: the experts' projections are stored in different dtypes")
         # one tensor per projection, [experts, rows, columns]: a kernel finds an expert's weights by its number
-        self.gate, self.up, self.down = (torch.stack([tensors[en[k]] for en in per]).contiguous() for k in ("gate", "up", "down"))
+        stacked = {k: torch.stack([tensors[en[k]] for en in per]).contiguous() for k in kinds}
+        self.gate, self.up, self.down = stacked.get("gate"), stacked["up"], stacked["down"]
         if self.shared is not None:
             self.shared.bind(tensors)
 
@@ -187,27 +218,29 @@ class MixtureMLP(FeedForward):
         ops = self.rt.ops
         pending = self.shared.forward(x, residual) if self.shared is not None else None
         logits = ops.linear(x, self.router, out_dtype=torch.float32, defer=True)  # few rows: partial sums, added by the routing
-        ids, weights = ops.moe_route(logits, self.bias, self.top)
-        xe = ops.cast(x, self.gate.dtype)  # experts stored in 32-bit compute in 32-bit
+        ids, weights = ops.moe_route(logits, self.bias, self.top, self.scoring, self.groups, self.keep_groups)
+        xe = ops.cast(x, self.up.dtype)  # experts stored in 32-bit compute in 32-bit
         ops.moe_experts(xe, ids, weights, self.gate, self.up, self.down, self.activation, residual)
         return pending
 
     def parameters_bytes(self) -> int:
         """What one token reads: the router, its ``top`` experts and the shared expert (a step of several tokens reads up
         to ``top`` experts more per token)."""
-        per_expert = sum(t[0].numel() * t.element_size() for t in (self.gate, self.up, self.down))
+        per_expert = sum(t[0].numel() * t.element_size() for t in (self.gate, self.up, self.down) if t is not None)
         own = self.router.numel() * self.router.element_size() + self.top * per_expert
         return own + (self.shared.parameters_bytes() if self.shared is not None else 0)
 
     def step_read_bytes(self, tokens: int) -> int:
         """The router, the shared expert and the experts that ``tokens`` tokens are expected to choose between them when
         every choice of ``top`` is as likely as any other: ``E (1 - (1 - top / E) ** tokens)`` experts."""
-        per_expert = sum(t[0].numel() * t.element_size() for t in (self.gate, self.up, self.down))
-        distinct = self.num_experts * (1.0 - (1.0 - self.top / self.num_experts) ** max(1, tokens))
+        per_expert = sum(t[0].numel() * t.element_size() for t in (self.gate, self.up, self.down) if t is not None)
+        distinct = self.num_experts * (1.0 - (1.0 - self.top / self.outputs) ** max(1, tokens))
         own = self.router.numel() * self.router.element_size() + int(round(distinct * per_expert))
         return own + (self.shared.parameters_bytes() if self.shared is not None else 0)
 
     def flops(self, rows) -> int:
         tokens = sum(n for n, _ in rows)
-        own = 2 * tokens * self.hidden * self.num_experts + 2 * tokens * self.top * 3 * self.hidden * self.inter
+        products = 3 if self.gated else 2
+        chosen = self.top * self.num_experts / self.outputs  # identity experts multiply nothing
+        own = 2 * tokens * self.hidden * self.outputs + int(2 * tokens * chosen * products * self.hidden * self.inter)
         return own + (self.shared.flops(rows) if self.shared is not None else 0)

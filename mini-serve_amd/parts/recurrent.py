@@ -7,6 +7,11 @@ slots; they differ in where ``a`` and ``b`` come from and in what happens to ``o
 
 * ``decay_linear_attention``: ``q, k, v = silu(W h)``; ``a`` is a constant per head (``decay``), ``b = 1``; the
   concatenated heads are RMS-normed together (weight ``norm``), multiplied by ``sigmoid(W_g h)`` and projected.
+  Options, whose defaults give that layer: ``activation`` (``"silu"`` or None: q, k, v as projected), ``position`` (a
+  position encoding that turns q and k, in float32, before the recurrence), ``k_scale`` (k is multiplied by it, behind
+  the rotation), ``norm_group`` (``"row"``: one norm over the concatenated heads; ``"head"``: one per head),
+  ``norm_weight`` (False: a bare division by the root mean square, no ``norm`` tensor), ``gate_activation``
+  (``"sigmoid"`` or ``"silu"``).
 * ``mlstm``: ``q = W_q h / sqrt(dim)``, ``k``, ``v`` plain; a log input gate and a log forget gate per head, each
   bounded by a soft cap (``cap tanh(z / cap)``, the forget gate then through a log-sigmoid), a running maximum that
   keeps the exponentials in range, and a normaliser vector ``n``; each head's output is divided by its root mean
@@ -14,6 +19,14 @@ slots; they differ in where ``a`` and ``b`` come from and in what happens to ``o
 
 All projections of a mixer are one matrix product over row-concatenated weights whose float32 result the recurrence
 kernel reads in place (activation, scale and gates are applied on the way in).
+
+* ``wkv``: the same state with a decay per key channel and token and a bonus for the current token,
+  ``o_t = (S_(t-1) + diag(u) k_t v_t^T)^T r_t``, then ``S_t = diag(w_t) S_(t-1) + k_t v_t^T``. Each of r, k, v, the gate and
+  the decay reads its own blend of the token's input and the previous token's, ``h + (h' - h) mu_s`` (``h' = 0`` for a
+  sequence's first token; a request's last input is part of its state); ``w = exp(-exp(W_w2 tanh(W_w1 mix_w) + w0))``;
+  each head's output is divided by its root mean square, the heads are concatenated, multiplied by a weight and by
+  ``silu(W_g mix_g)`` and projected. Its five products read five different inputs, so they stay five products; they
+  write into the columns of one float32 matrix that the kernels behind them read side by side.
 """
 
 from __future__ import annotations
@@ -59,17 +72,17 @@ class _RecurrentMixer(Mixer):
             at += t.shape[0]
         self.proj = torch.cat(parts, dim=0).contiguous()
         self.o = tensors[self.names["o"]]
-        self.norm = tensors[self.names["norm"]]
+        self.norm = tensors[self.names["norm"]] if self.names["norm"] in tensors else None
 
-    def _finish(self, o, x32, group, residual):
+    def _finish(self, o, x32, group, residual, gate_activation: str = "sigmoid"):
         ops = self.rt.ops
         n = self.heads * self.value_dim
         gate = x32[:, self.columns["g"] : self.columns["g"] + n]
-        y = ops.group_rmsnorm_gate(o, group, self.norm, gate, self.eps, self.rt.dtype)
+        y = ops.group_rmsnorm_gate(o, group, self.norm, gate, self.eps, self.rt.dtype, gate_activation)
         return ops.linear(y, self.o, accumulate_into=residual, defer=True)
 
     def parameters_bytes(self) -> int:
-        return sum(t.numel() * t.element_size() for t in (self.proj, self.o, self.norm))
+        return sum(t.numel() * t.element_size() for t in (self.proj, self.o, self.norm) if t is not None)
 
     def flops(self, rows) -> int:
         tokens = sum(n for n, _ in rows)
@@ -91,14 +104,29 @@ class DecayLinearAttention(_RecurrentMixer):
             raise ValueError(f"decays must lie in [0, 1], got {decay}")
         self.decay = torch.tensor(decay, dtype=torch.float32, device=rt.device) if rt is not None else None
         self.chunks = min(decay) > 1e-30  # the chunked kernels work with the decays' logarithms
+        self.activation = spec.get("activation", "silu")
+        self.k_scale = float(spec.get("k_scale", 1.0))
+        self.norm_group = spec.get("norm_group", "row")
+        self.gate_activation = spec.get("gate_activation", "sigmoid")
+        if self.activation not in (None, "silu"):
+            raise NotImplementedError(f"activation {self.activation!r} of q, k and v: None or 'silu'")
+        if self.norm_group not in ("row", "head"):
+            raise ValueError(f"norm_group {self.norm_group!r}: 'row' or 'head'")
+        if rt is not None and self.gate_activation not in rt.ops.GATE_ACTIVATIONS:
+            raise NotImplementedError(f"gate activation {self.gate_activation!r}: one of {sorted(rt.ops.GATE_ACTIVATIONS)}")
+        pos = spec.get("position") or PartSpec("none")
+        self.position = part_class("position", pos)(pos, rt)
 
     @classmethod
     def tensors(cls, spec: PartSpec) -> dict[str, TensorSpec]:
         n = _named(spec, cls.NAMES)
         w, h, d = int(spec["hidden_size"]), int(spec["num_heads"]), int(spec["head_dim"])
         e = int(spec.get("value_dim") or d)
-        return {n["q"]: TensorSpec((h * d, w)), n["k"]: TensorSpec((h * d, w)), n["v"]: TensorSpec((h * e, w)),
-                n["g"]: TensorSpec((h * e, w)), n["o"]: TensorSpec((w, h * e)), n["norm"]: TensorSpec((h * e,), init="ones")}
+        out = {n["q"]: TensorSpec((h * d, w)), n["k"]: TensorSpec((h * d, w)), n["v"]: TensorSpec((h * e, w)),
+               n["g"]: TensorSpec((h * e, w)), n["o"]: TensorSpec((w, h * e))}
+        if spec.get("norm_weight", True):
+            out[n["norm"]] = TensorSpec((h * e,), init="ones")
+        return out
 
     def bind(self, tensors) -> None:
         self._fuse(tensors, ("q", "k", "v", "g"))
@@ -109,9 +137,17 @@ class DecayLinearAttention(_RecurrentMixer):
     def forward(self, x, batch, cache, state, residual):
         ops = self.rt.ops
         x32 = ops.linear(x, self.proj, out_dtype=torch.float32)
+        rot = self.position.rotation(batch)
+        if rot is not None or self.k_scale != 1.0:
+            if rot is not None and self.activation is not None:
+                raise NotImplementedError("a rotation of q and k goes with q and k as projected (activation None)")
+            table, pairing = (rot.table, rot.pairing) if rot is not None else (None, "halves")
+            ops.rotate_columns_(x32, self.columns["q"], self.heads, self.dim, table, pairing, 1.0)
+            ops.rotate_columns_(x32, self.columns["k"], self.heads, self.dim, table, pairing, self.k_scale)
         o = ops.gated_recurrence(x32, self.columns, self.heads, self.dim, self.value_dim, batch, state, mode="decay",
-                                 activation="silu", decay=self.decay, chunks=self.chunks)
-        return self._finish(o, x32, self.heads * self.value_dim, residual)
+                                 activation=self.activation, decay=self.decay, chunks=self.chunks)
+        group = self.value_dim if self.norm_group == "head" else self.heads * self.value_dim
+        return self._finish(o, x32, group, residual, self.gate_activation)
 
 
 @register("mixer", "mlstm")
@@ -153,6 +189,86 @@ class MLSTM(_RecurrentMixer):
 
     def parameters_bytes(self) -> int:
         return super().parameters_bytes() + sum(t.numel() * t.element_size() for t in (self.i_bias, self.f_bias))
+
+
+@register("mixer", "wkv")
+class WKV(_RecurrentMixer):
+    NAMES = {"r": "r", "k": "k", "v": "v", "g": "g", "w1": "w1", "w2": "w2", "w0": "w0", "u": "u", "o": "o", "norm": "norm",
+             "mu_r": "mu.r", "mu_k": "mu.k", "mu_v": "mu.v", "mu_g": "mu.g", "mu_w": "mu.w"}
+    BLENDS = ("r", "k", "v", "g", "w")  # the order of the blends; the decay's first step is the fifth product
+
+    def __init__(self, spec: PartSpec, rt):
+        super().__init__(spec, rt)
+        if self.value_dim != self.dim:
+            raise ValueError(f"wkv heads have keys and values of one size, not {self.dim} / {self.value_dim}")
+        # the width of the decay's first step: a configuration may state it; else the checkpoint's tensors say it
+        self.rank = int(spec["decay_rank"]) if spec.get("decay_rank") else None
+        self.ld = 0
+        self.mu = self.weights = self.w2t = self.w0 = self.u = None
+
+    @classmethod
+    def tensors(cls, spec: PartSpec) -> dict[str, TensorSpec]:
+        n = _named(spec, cls.NAMES)
+        w, h, d = int(spec["hidden_size"]), int(spec["num_heads"]), int(spec["head_dim"])
+        r = int(spec["decay_rank"]) if spec.get("decay_rank") else None
+        free = None if r is not None else max(8, min(64, w // 16))
+        out = {n[k]: TensorSpec((h * d, w)) for k in ("r", "k", "v", "g")}
+        out.update({n[f"mu_{k}"]: TensorSpec((w,), init="uniform") for k in cls.BLENDS})
+        out.update({n["w1"]: TensorSpec((r, w), free=free), n["w2"]: TensorSpec((h * d, r), free=free),
+                    n["w0"]: TensorSpec((h * d,), init="uniform"),
+                    n["u"]: TensorSpec((h, d), init="uniform"), n["norm"]: TensorSpec((h * d,), init="ones"),
+                    n["o"]: TensorSpec((w, h * d))})
+        return out
+
+    def bind(self, tensors) -> None:
+        n = self.names
+        self.weights = [tensors[n[k]] for k in ("r", "k", "v", "g", "w1")]
+        if len({t.dtype for t in self.weights}) != 1:
+            raise ValueError(f"{n['r']} and its neighbours are stored in different dtypes")
+        dtype = self.weights[0].dtype
+        self.rank = self.weights[4].shape[0]
+        if tensors[n["w2"]].shape[1] != self.rank:
+            raise ValueError(f"{n['w1']} has {self.rank} rows, {n['w2']} {tensors[n['w2']].shape[1]} columns")
+        if not 1 <= self.rank <= self.rt.ops.CHANNEL_DECAY_MAX_RANK:
+            raise ValueError(f"{n['w1']}: {self.rank} rows; the decay's kernel takes 1..{self.rt.ops.CHANNEL_DECAY_MAX_RANK}")
+        at = 0
+        width = self.heads * self.dim
+        for k, cols in (("q", width), ("k", width), ("v", width), ("g", width), ("a", self.rank)):  # q: the receptance; a: the decay's first step
+            self.columns[k] = at
+            at += -(-cols // 4) * 4  # every product's columns start 16-byte aligned
+        self.ld = at
+        self.mu = torch.stack([tensors[n[f"mu_{k}"]].to(dtype) for k in self.BLENDS]).contiguous()
+        self.w2t = tensors[n["w2"]].t().contiguous()  # [rank, channels]: a thread per channel reads side by side
+        self.w0 = tensors[n["w0"]].to(self.w2t.dtype).contiguous()
+        self.u = tensors[n["u"]].to(torch.float32).contiguous()
+        self.o, self.norm = tensors[n["o"]], tensors[n["norm"]]
+
+    def state_need(self) -> StateNeed:
+        return StateNeed((StateTensor("S", (self.heads, self.dim, self.dim), "float32"),
+                          StateTensor("shift", (self.hidden,), "float32")))
+
+    def forward(self, x, batch, cache, state, residual):
+        ops = self.rt.ops
+        c, n = self.columns, self.heads * self.dim
+        blends = ops.token_shift_mix(ops.cast(x, self.mu.dtype), self.mu, state["shift"], batch)
+        x32 = torch.empty((x.shape[0], self.ld), dtype=torch.float32, device=x.device)
+        for i, (k, w) in enumerate(zip(("q", "k", "v", "g", "a"), self.weights)):
+            ops.linear(blends[i], w, out=x32[:, c[k] : c[k] + w.shape[0]])
+        decay = ops.channel_decay(x32, c["a"], self.w2t, self.w0)
+        o = ops.gated_recurrence(x32, c, self.heads, self.dim, self.dim, batch, state, mode="wkv", channel_decay=decay, bonus=self.u)
+        y = ops.group_rmsnorm_gate(o, self.dim, self.norm, x32[:, c["g"] : c["g"] + n], self.eps, self.rt.dtype, "silu")
+        return ops.linear(y, self.o, accumulate_into=residual, defer=True)
+
+    def parameters_bytes(self) -> int:
+        ts = self.weights + [self.mu, self.w2t, self.w0, self.u, self.o, self.norm]
+        return sum(t.numel() * t.element_size() for t in ts)
+
+    def flops(self, rows) -> int:
+        tokens = sum(n for n, _ in rows)
+        n = self.heads * self.dim
+        rank = self.rank or 0
+        linear = 2 * tokens * self.hidden * (4 * n + rank) + 2 * tokens * rank * n + 2 * tokens * n * self.hidden
+        return linear + 6 * tokens * self.heads * self.dim * self.dim
 
 
 @register("mixer", "normed_pair")

@@ -85,7 +85,7 @@ def load_weights(
                     unexpected.append(name)
                     continue
                 shape = tuple(sf.get_slice(name).get_shape())
-                if shape != ts.shape:
+                if not ts.fits(shape):
                     mismatched.append(f"{name}: {shape} != {ts.shape}")
                     continue
                 try:

@@ -48,20 +48,20 @@ def random_tensors(
         if ts.optional:
             continue
         if ts.kind == "int":
-            out[name] = torch.randint(0, ts.high, ts.shape, generator=gen, dtype=torch.int32, device=device)
+            out[name] = torch.randint(0, ts.high, ts.drawn_shape(), generator=gen, dtype=torch.int32, device=device)
             continue
         if ts.init == "ones":
             if init.norm_range is None:
-                t = torch.ones(ts.shape, **f32)
+                t = torch.ones(ts.drawn_shape(), **f32)
             else:
                 lo, hi = init.norm_range
-                t = torch.rand(ts.shape, generator=gen, **f32) * (hi - lo) + lo
+                t = torch.rand(ts.drawn_shape(), generator=gen, **f32) * (hi - lo) + lo
         elif ts.init == "zeros":
-            t = torch.zeros(ts.shape, **f32)
+            t = torch.zeros(ts.drawn_shape(), **f32)
         elif ts.init == "uniform":
-            t = (torch.rand(ts.shape, generator=gen, **f32) * 2 - 1) * init.std
+            t = (torch.rand(ts.drawn_shape(), generator=gen, **f32) * 2 - 1) * init.std
         else:
-            t = torch.randn(ts.shape, generator=gen, **f32) * init.std
+            t = torch.randn(ts.drawn_shape(), generator=gen, **f32) * init.std
         out[name] = t.to(torch.bfloat16).to(dtype)
     return out
 
