@@ -146,6 +146,27 @@ def _reselorn_tiny() -> dict:
 PRESETS["reselorn-tiny"] = _reselorn_tiny()
 
 
+def _zigelorn_tiny() -> dict:
+    """Six layers that hold every part of the architecture once: the three mixers, a dense feed-forward, a mixture with
+    identity experts and groups, a layer without a feed-forward, and a layer that runs another's weights over a state of its own."""
+    slowed = {"base": 3000.0, "dims": 12, "scaling": {"factor": 8.0, "original": 48, "fast": 6.0, "slow": 0.5}}
+    attention = {"type": "attention", "mixer": {"heads": 4, "kv_heads": 2, "dim": 24, "vdim": 24, "scale": 24 ** -0.5, "rot": slowed,
+                                                "mask": {"size": 24}},
+                 "mlp": {"kind": "moe", "router": {"experts": 6, "identity": 2, "top": 3, "groups": {"count": 4, "keep": 2}},
+                         "expert": {"ff": 48}}}
+    wkv = {"type": "wkv", "mixer": {"heads": 3, "dim": 32, "rank": 12}, "mlp": {"kind": "dense", "ff": 160}}
+    retention = {"type": "retention", "mixer": {"heads": 3, "dim": 16, "vdim": 32, "decay": [0.9, 0.97, 0.995],
+                                                "rot": {"base": 100.0, "dims": 16}}, "mlp": None}
+    return {
+        "architecture": "Zigelorn", "vocab": 311, "width": 96, "norm": {"eps": 1e-5},
+        "layers": [wkv, attention, retention, dict(copy.deepcopy(attention), weights_of=1), dict(copy.deepcopy(wkv), weights_of=0),
+                   {"type": "retention", "mixer": {"heads": 2, "dim": 8, "vdim": 8, "decay": [0.5, 1.0]}, "mlp": {"kind": "dense", "ff": 64}}],
+    }
+
+
+PRESETS["zigelorn-tiny"] = _zigelorn_tiny()
+
+
 def preset(name: str) -> dict:
     try:
         return copy.deepcopy(PRESETS[name])

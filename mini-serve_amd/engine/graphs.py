@@ -53,7 +53,7 @@ class DecodeGraphs:
 
     def _key(self, rows):
         g = next(b for b in self.buckets if b >= len(rows))
-        need = max(max(t.num_entries for t in r.cache.tables) for r in rows)
+        need = max(max((t.num_entries for t in r.cache.tables), default=0) for r in rows)  # (a model may keep no pages at all)
         w = self.MIN_WIDTH
         while w < need:
             w *= 2

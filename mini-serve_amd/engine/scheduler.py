@@ -157,9 +157,9 @@ class Scheduler:
             if r.cache is None:
                 continue  # everything sampled: it holds nothing and runs no more
             if r.state is RequestState.PREFILL:
-                need += self.cache.outstanding(r.cache, r.seq_len + 1, self._step_of(r))
+                need += np.asarray(self.cache.outstanding(r.cache, r.seq_len + 1, self._step_of(r)), dtype=np.int64)  # (a model may keep no pages at all)
             elif r.decodes:
-                need += self.cache.pages_needed(r.cache, 1)
+                need += np.asarray(self.cache.pages_needed(r.cache, 1), dtype=np.int64)
         return need
 
     def _free(self) -> np.ndarray:
@@ -227,7 +227,7 @@ class Scheduler:
                 if rows and n > budget:
                     break  # only the first prompt of a step may exceed the budget
             handle = self.cache.acquire()
-            need = self.cache.outstanding(handle, req.seq_len + 1, self._step_of(req))
+            need = np.asarray(self.cache.outstanding(handle, req.seq_len + 1, self._step_of(req)), dtype=np.int64)
             if (need > self._free() - self._may_draw(self.running)).any():
                 self.cache.release(handle)  # nothing stays behind a refused admission
                 break

@@ -216,8 +216,9 @@ def _sub(weights, prefix):
     return {k[len(prefix):]: v for k, v in weights.items() if k.startswith(prefix)}
 
 
-def forward(cfg, weights, tokens, return_layers=False):
-    """Logits ``[T, vocab]`` of one sequence (and, asked for, the stream after every layer ``[layers, T, W]``)."""
+def forward(cfg, weights, tokens, return_layers=False, watch=None):
+    """Logits ``[T, vocab]`` of one sequence (and, asked for, the stream after every layer ``[layers, T, W]``).
+    ``watch(i, x)`` is shown the stream that layer ``i``'s feed-forward norm reads."""
     eps = cfg["norm"]["eps"]
     tokens = np.asarray(tokens)
     positions = np.arange(len(tokens))
@@ -239,6 +240,8 @@ def forward(cfg, weights, tokens, return_layers=False):
         mlp = layer.get("mlp")
         if mlp:
             wf = _sub(weights, p + "mlp.")
+            if watch is not None:
+                watch(i, x)
             h = one_plus_norm(x, weights[p + "norm2"], eps)
             y = dense_ff(h, wf) if mlp["kind"] == "dense" else mixture_ff(h, wf, mlp)
             x = x + one_plus_norm(y, weights[p + "norm2b"], eps)
