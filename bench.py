@@ -25,8 +25,9 @@ with its share of the roofline), ``measured_peaks`` (what this box gives a strea
 and the engine's bfloat16 product) and ``sidecar`` (device, clocks and power while the headline point
 ran, versions, commit, the engine's effective configuration).
 
-``--design kakunex`` (or ``fimolix``, ``reselorn``) measures something else and leaves the above as it is: prefill and decode
-throughput of that architecture beside Qwen3 models of equal size (``miniserve_amd/measurement/designs.py``), one JSON line.
+``--design kakunex`` (or ``fimolix``, ``reselorn``, ``zigelorn``) measures something else and leaves the above as it is: prefill
+and decode throughput of that architecture beside Qwen3 models of equal size (Zigelorn: beside Kakunex models, the
+other design of windowed attention and linear recurrences; ``miniserve_amd/measurement/designs.py``), one JSON line.
 
 Peaks: MI355X's published 8 TB/s HBM and 2.5 PFLOP/s dense bf16 (157.3 TFLOP/s float32).
 """
@@ -74,19 +75,20 @@ def main() -> int:
     ap.add_argument("--prefill-tokens", type=int, default=2048, help="tokens of the timed prefill step")
     ap.add_argument("--prefill-cached", type=int, default=0,
                     help="tokens of the same sequence already in the cache when the timed step runs (fed untimed, 2,048 a step)")
-    ap.add_argument("--design", choices=("kakunex", "fimolix", "reselorn"), default=None,
-                    help="instead of the workload above: prefill and decode of this architecture beside Qwen3 of equal size")
+    ap.add_argument("--design", choices=("kakunex", "fimolix", "reselorn", "zigelorn"), default=None,
+                    help="instead of the workload above: prefill and decode of this architecture beside Qwen3 (zigelorn: Kakunex) of equal size")
     ap.add_argument("--shapes", default=None, help="with --design: the shapes to run, with commas between them (default: all)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
     if args.design:
-        from miniserve_amd.measurement.designs import compare
+        from miniserve_amd.measurement.designs import BESIDE, compare
 
+        beside = BESIDE.get(args.design, "qwen3")
         got = compare(args.design, args.shapes.split(",") if args.shapes else None, args.dtype, args.prefill_tokens, args.batch,
                       2048, args.steps, args.warmup, say=say)
-        print(json.dumps({"metric": f"prefill and decode tok/s of {args.design} beside qwen3 at equal sizes", "unit": "tok/s",
+        print(json.dumps({"metric": f"prefill and decode tok/s of {args.design} beside {beside} at equal sizes", "unit": "tok/s",
                           "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
                           "data": "synthetic (random weights, random token ids)", "prefill_tokens": args.prefill_tokens,
                           "decode_batch": args.batch, "decode_context": 2048, "shapes": got}))

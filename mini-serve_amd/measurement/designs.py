@@ -1,6 +1,6 @@
 """Prefill and decode throughput of one architecture beside another of equal size: random weights, layers of the
-sizes real models have, the same step function for both. ``bench.py --design kakunex`` (or ``fimolix``, ``reselorn``)
-prints what this returns.
+sizes real models have, the same step function for both. ``bench.py --design kakunex`` (or ``fimolix``, ``reselorn``,
+``zigelorn``) prints what this returns.
 
 A *shape* fixes what the two share: width, query and key/value heads of 128 elements, feed-forward width, window,
 layers, vocabulary. The Kakunex model of a shape repeats (parallel, parallel, parallel, mlstm): window attention that
@@ -17,7 +17,14 @@ per token, inside the shape's window.
 The Reselorn model of a shape has the shape's heads of 128 elements (half of them rotated, slowed frequencies), a sink
 per head, the shape's window and blended values in every layer; its first layer has the shape's dense feed-forward, the
 others a mixture of 32 experts of an eighth of that width, of which a token runs 4, beside a shared expert of half the
-width: a token multiplies as much as in the Qwen3 layer, the weights are 4.5 times the layer's."""
+width: a token multiplies as much as in the Qwen3 layer, the weights are 4.5 times the layer's.
+
+The Zigelorn model of a shape repeats (wkv, attention, retention, wkv): the attention has the shape's heads of 128 (half
+of each rotated, slowed frequencies) inside the shape's window, the retention as many heads of 128 x 128 with rotated
+queries and keys, the wkv layers ``width / 64`` heads of 64 x 64 with a decay projection 64 wide. Feed-forwards alternate:
+a dense one without a gate, 1.5 times the shape's width (as many multiplications as the gated one of the shape), and a
+mixture of 28 experts of a quarter of that beside 4 identity experts, 8 groups of which 4 are kept, 4 chosen. It is
+measured beside the Kakunex model of the shape, the other design of windowed attention and linear recurrences."""
 
 from __future__ import annotations
 
@@ -90,7 +97,24 @@ def reselorn_config(s: dict) -> dict:
     return {"architecture": "Reselorn", "vocab": s["vocab"], "width": s["width"], "norm": {"eps": 1e-6}, "layers": layers}
 
 
-DESIGNS = {"kakunex": kakunex_config, "fimolix": fimolix_config, "reselorn": reselorn_config, "qwen3": qwen3_config}
+def zigelorn_config(s: dict) -> dict:
+    rot = {"base": 1e6, "dims": HEAD // 2, "scaling": {"factor": 8.0, "original": 4096, "fast": 32.0, "slow": 1.0}}
+    attention = {"heads": s["heads"], "kv_heads": s["kv_heads"], "dim": HEAD, "vdim": HEAD, "scale": HEAD ** -0.5, "rot": rot,
+                 "mask": {"size": s["window"]}}
+    decays = [1.0 - 2.0 ** -(5 + 6 * i / max(1, s["heads"] - 1)) for i in range(s["heads"])]
+    retention = {"heads": s["heads"], "dim": HEAD, "vdim": HEAD, "decay": decays, "rot": {"base": 1e6, "dims": HEAD}}
+    wkv = {"heads": s["width"] // 64, "dim": 64, "rank": 64}
+    ff = s["ff"] * 3 // 2
+    dense = {"kind": "dense", "ff": ff}
+    mixture = {"kind": "moe", "router": {"experts": 28, "identity": 4, "top": 4, "groups": {"count": 8, "keep": 4}}, "expert": {"ff": ff // 4}}
+    kinds = (("wkv", wkv, dense), ("attention", attention, mixture), ("retention", retention, dense), ("wkv", wkv, mixture))
+    layers = [{"type": kinds[i % 4][0], "mixer": dict(kinds[i % 4][1]), "mlp": dict(kinds[i % 4][2])} for i in range(s["layers"])]
+    return {"architecture": "Zigelorn", "vocab": s["vocab"], "width": s["width"], "norm": {"eps": 1e-6}, "layers": layers}
+
+
+DESIGNS = {"kakunex": kakunex_config, "fimolix": fimolix_config, "reselorn": reselorn_config, "zigelorn": zigelorn_config,
+           "qwen3": qwen3_config}
+BESIDE = {"zigelorn": "kakunex"}  # the model a design is measured beside (default: qwen3)
 
 
 def measure(config: dict, dtype: str, prefill_tokens: int, batch: int, context: int, steps: int, warmup: int, say=lambda m: None) -> dict:
@@ -154,8 +178,9 @@ def measure(config: dict, dtype: str, prefill_tokens: int, batch: int, context: 
 
 
 def compare(design: str, shapes=None, dtype: str = "bfloat16", prefill_tokens: int = 2048, batch: int = 8, context: int = 2048,
-            steps: int = 32, warmup: int = 8, beside: str = "qwen3", say=lambda m: None) -> dict:
+            steps: int = 32, warmup: int = 8, beside: str | None = None, say=lambda m: None) -> dict:
     """``{shape: {design: figures, beside: figures}}`` for the named shapes (all by default)."""
+    beside = beside or BESIDE.get(design, "qwen3")
     out = {}
     for name in shapes or sorted(SHAPES):
         s = SHAPES[name]

@@ -16,6 +16,7 @@ implementation, and the comparison would say nothing about the kernels."""
 
 from __future__ import annotations
 
+import copy
 from pathlib import Path
 
 import numpy as np
@@ -51,7 +52,7 @@ def wkv(heads, dim, rank, mlp=None, **more):
 
 def again(layers, j):
     """Layer ``j`` of ``layers`` once more: its weights, a cache and state of its own."""
-    out = {k: v for k, v in layers[j].items()}
+    out = copy.deepcopy(layers[j])
     out["weights_of"] = j
     return out
 
