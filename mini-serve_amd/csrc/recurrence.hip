@@ -7,7 +7,7 @@
 //       m_t = max(f_t + m_(t-1), i_t) (m starts at 0) that keeps the exponentials in range:
 //       a_t = exp(f_t + m_(t-1) - m_t), b_t = exp(i_t - m_t); a vector n_t = a_t n_(t-1) + b_t k_t beside S;
 //       o_t = S_t^T q_t / (max(|n_t . q_t|, exp(-m_t)) + 1e-6).
-//   MS_REC_WKV: a decay per key channel and token, w_t [D] (row t of the float32 matrix `w`, columns h D ..), and a bonus
+//   MS_REC_WKV: a decay per key channel and token, w_t [D] (its logarithm is row t of the float32 matrix `w`, columns h D ..), and a bonus
 //       u [H, D] that only the current token gets: o_t = (S_(t-1) + diag(u) k_t v_t^T)^T q_t, and only then
 //       S_t = diag(w_t) S_(t-1) + k_t v_t^T.
 // q, k, v (and the gates' inputs) are columns of one float32 matrix x [tokens, ld] (the layer's projections);
@@ -44,7 +44,7 @@ struct RecurrenceArgs {
   const int* starts;
   const int* state_slots;
   float* out;
-  const float* w;  // MS_REC_WKV: the decays [tokens, ld_w], head h's D channels from column h D on
+  const float* w;  // MS_REC_WKV: the decays' logarithms [tokens, ld_w], head h's D channels from column h D on
   int ld_w;
   const float* u;  // MS_REC_WKV: the bonus [H, D]
 };
@@ -105,7 +105,7 @@ __global__ __launch_bounds__(256) void gated_recurrence_kernel(RecurrenceArgs a,
       kd = rec_act(xr[a.k_off + h * D + tid], a.act);
       qs[buf][tid] = qd;
       ks[buf][tid] = kd;
-      if (wkv) ws[buf][tid] = a.w[(size_t)t * a.ld_w + h * D + tid];
+      if (wkv) ws[buf][tid] = expf(a.w[(size_t)t * a.ld_w + h * D + tid]);
     }
     if (gates) {
       nv = fs * nv + is * kd;  // threads beyond D carry zeros

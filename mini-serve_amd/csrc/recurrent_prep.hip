@@ -83,13 +83,15 @@ extern "C" int ms_token_shift_mix(const void* h, const void* mu, void* out, int 
 }
 
 // ---------------------------------------------------------------------------------------------
-// out[t][c] = exp(-exp(sum_r w2t[r][c] tanh(a[t][col + r]) + w0[c])), c < C, r < R: the decay of channel c at token t.
+// out[t][c] = exp(-exp(sum_r w2t[r][c] tanh(a[t][col + r]) + w0[c])), c < C, r < R: the decay of channel c at token t; or,
+// as_log, its logarithm -exp(...), which a sum over tokens keeps sharp where the decay is next to one.
 // a: float32 [tokens, lda] (the first step's projection); w2t: the second step's weight transposed, [R, C]; w0 [C].
 // Float32 throughout, the sum in ascending r. One block per token; tanh(a[t]) goes through LDS.
 #define DECAY_MAX_RANK 1024
 template <typename TW>
 __global__ __launch_bounds__(256) void channel_decay_kernel(const float* __restrict__ a, int lda, int col, const TW* __restrict__ w2t,
-                                                            const TW* __restrict__ w0, float* __restrict__ out, int C, int R) {
+                                                            const TW* __restrict__ w0, float* __restrict__ out, int C, int R,
+                                                            int as_log) {
   __shared__ float th[DECAY_MAX_RANK];
   const int t = blockIdx.x;
   for (int r = threadIdx.x; r < R; r += 256) th[r] = tanhf(a[(size_t)t * lda + col + r]);
@@ -97,16 +99,17 @@ __global__ __launch_bounds__(256) void channel_decay_kernel(const float* __restr
   for (int c = threadIdx.x; c < C; c += 256) {
     float z = 0.f;
     for (int r = 0; r < R; ++r) z = fmaf(to_f32(w2t[(size_t)r * C + c]), th[r], z);
-    out[(size_t)t * C + c] = expf(-expf(z + to_f32(w0[c])));
+    const float l = -expf(z + to_f32(w0[c]));
+    out[(size_t)t * C + c] = as_log ? l : expf(l);
   }
 }
 
 extern "C" int ms_channel_decay(const float* a, int lda, int col, const void* w2t, const void* w0, int w_is_bf16, float* out,
-                                int tokens, int C, int R, hipStream_t st) {
+                                int tokens, int C, int R, int as_log, hipStream_t st) {
   if (tokens <= 0) return MS_OK;
   if (a == nullptr || w2t == nullptr || w0 == nullptr || out == nullptr || C <= 0 || R <= 0 || col < 0 || col + R > lda) return MS_BAD_ARG;
   if (R > DECAY_MAX_RANK) return MS_UNSUPPORTED;
-  if (w_is_bf16) channel_decay_kernel<bf16><<<tokens, 256, 0, st>>>(a, lda, col, (const bf16*)w2t, (const bf16*)w0, out, C, R);
-  else channel_decay_kernel<float><<<tokens, 256, 0, st>>>(a, lda, col, (const float*)w2t, (const float*)w0, out, C, R);
+  if (w_is_bf16) channel_decay_kernel<bf16><<<tokens, 256, 0, st>>>(a, lda, col, (const bf16*)w2t, (const bf16*)w0, out, C, R, as_log);
+  else channel_decay_kernel<float><<<tokens, 256, 0, st>>>(a, lda, col, (const float*)w2t, (const float*)w0, out, C, R, as_log);
   return launch_status();
 }

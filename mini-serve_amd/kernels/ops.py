@@ -39,7 +39,11 @@ _SIGNATURES = {
                             _c_int, _c_void, _c_int, _c_void, _c_void],
     "ms_rotate_columns": [_c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void, _c_int, _c_int, _c_float, _c_void],
     "ms_token_shift_mix": [_c_void, _c_void, _c_void, _c_int, _c_void, _c_void, _c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_void],
-    "ms_channel_decay": [_c_void, _c_int, _c_int, _c_void, _c_void, _c_int, _c_void, _c_int, _c_int, _c_int, _c_void],
+    "ms_channel_decay": [_c_void, _c_int, _c_int, _c_void, _c_void, _c_int, _c_void, _c_int, _c_int, _c_int, _c_int, _c_void],
+    "ms_wkv_chunked": [_c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void, _c_int, _c_void, _c_void, _c_void, _c_void, _c_void,
+                       _c_void, _c_int, _c_int, _c_void, _c_void, _c_void],
+    "ms_wkv_chunk_tokens": [],
+    "ms_wkv_chunk_max_dim": [],
     "ms_gated_recurrence_chunked": [_c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
                                     _c_float, _c_float, _c_void, _c_void, _c_void, _c_int, _c_void, _c_void, _c_void, _c_void, _c_void,
                                     _c_void, _c_void, _c_int, _c_int, _c_void, _c_void, _c_void, _c_void],
@@ -1550,6 +1554,7 @@ DECODE_GENERIC_WAVES = 16  # waves that share a (token, head) in the float32 att
 RECURRENCE_MODES = {"decay": 0, "exp_gates": 1, "wkv": 2}
 RECURRENCE_MAX_DIM = 256
 RECURRENCE_CHUNKED_FROM = 16  # tokens of the longest row from which a step runs the chunked kernels
+WKV_CHUNKED_FROM = 16  # ... and from which the recurrence with a decay per channel does
 
 
 def gated_recurrence(x: torch.Tensor, columns: dict, heads: int, dim: int, value_dim: int, batch, state: dict, *,
@@ -1564,9 +1569,10 @@ def gated_recurrence(x: torch.Tensor, columns: dict, heads: int, dim: int, value
     each). ``activation`` (None or ``"silu"``) is applied to q, k and v; q is then scaled by ``q_scale``.
     ``mode="decay"``: ``a = decay[head]``, ``b = 1``. ``mode="exp_gates"``: capped exponential gates with a running
     maximum and a normaliser (the kernel's source states the formulas); ``state`` then also holds ``n`` and ``m``.
-    ``mode="wkv"``: a decay per key channel and token, ``channel_decay`` (float32 ``[T, heads * dim]``), and a ``bonus``
-    (float32 ``[heads, dim]``) for the current token alone: ``o_t = (S_(t-1) + diag(bonus) k_t v_t^T)^T q_t``, then
-    ``S_t = diag(channel_decay_t) S_(t-1) + k_t v_t^T``.
+    ``mode="wkv"``: a decay per key channel and token, given by its logarithm ``channel_decay`` (float32
+    ``[T, heads * dim]``, at most zero), and a ``bonus`` (float32 ``[heads, dim]``) for the current token alone:
+    ``o_t = (S_(t-1) + diag(bonus) k_t v_t^T)^T q_t``, then ``S_t = diag(exp(channel_decay_t)) S_(t-1) + k_t v_t^T``
+    (``dim == value_dim``). Rows of ``WKV_CHUNKED_FROM`` tokens or more run in chunks (head sizes up to 64).
     ``state["S"]``: float32 ``[slots, heads, dim, value_dim]``; rows with ``starts == 0`` begin from zero.
     Returns float32 ``[T, heads * value_dim]``.
 
@@ -1609,7 +1615,8 @@ def gated_recurrence(x: torch.Tensor, columns: dict, heads: int, dim: int, value
         if tuple(channel_decay.shape) != (t, heads * dim) or tuple(bonus.shape) != (heads, dim):
             raise ValueError(f"channel_decay {tuple(channel_decay.shape)} / bonus {tuple(bonus.shape)} do not fit {t} tokens of "
                              f"{heads} heads of {dim}")
-        chunks = False  # the chunked kernels know one decay per head and token
+        if dim != value_dim:
+            raise ValueError(f"wkv heads have keys and values of one size, not {dim} / {value_dim}")
     else:
         _dev(decay, "decay", F32, 1)
         if decay.shape[0] != heads:
@@ -1630,6 +1637,18 @@ def gated_recurrence(x: torch.Tensor, columns: dict, heads: int, dim: int, value
     bias = i_bias if i_bias is not None else f_bias
     lib = library()
     lens = getattr(batch, "row_lens", None)
+    if mode == "wkv":
+        if chunks and lens is not None and max(lens) >= WKV_CHUNKED_FROM and dim <= lib.ms_wkv_chunk_max_dim():
+            per = lib.ms_wkv_chunk_tokens()
+            n_chunks = sum(-(-n // per) for n in lens)
+            U = torch.empty((n_chunks, heads, dim * dim), dtype=F32, device=x.device)
+            G = torch.empty((n_chunks, heads, dim), dtype=F32, device=x.device)
+            _check(lib.ms_wkv_chunked(x.data_ptr(), ld, columns["q"], columns["k"], columns["v"], heads, dim, channel_decay.data_ptr(),
+                                      heads * dim, bonus.data_ptr(), S.data_ptr(), batch.row_start.data_ptr(), batch.starts.data_ptr(),
+                                      batch.state_slots.data_ptr(), out.data_ptr(), rows, n_chunks, U.data_ptr(), G.data_ptr(), _stream()),
+                   "wkv_chunked")
+            return out
+        chunks = False
     if (chunks and lens is not None and max(lens) >= RECURRENCE_CHUNKED_FROM
             and max(dim, value_dim) <= lib.ms_gated_recurrence_chunk_max_dim()):
         per = lib.ms_gated_recurrence_chunk_tokens()
@@ -1700,9 +1719,10 @@ def token_shift_mix(h: torch.Tensor, mu: torch.Tensor, carry: torch.Tensor, batc
 CHANNEL_DECAY_MAX_RANK = 1024  # DECAY_MAX_RANK in csrc/recurrent_prep.hip
 
 
-def channel_decay(a: torch.Tensor, col: int, w2t: torch.Tensor, w0: torch.Tensor) -> torch.Tensor:
+def channel_decay(a: torch.Tensor, col: int, w2t: torch.Tensor, w0: torch.Tensor, log: bool = False) -> torch.Tensor:
     """``exp(-exp(tanh(a[:, col : col + R]) @ w2t + w0))``: float32 ``[T, C]`` from the float32 ``a [T, >= col + R]``,
-    ``w2t [R, C]`` and ``w0 [C]`` (one dtype), float32 arithmetic, the sum in ascending ``r``."""
+    ``w2t [R, C]`` and ``w0 [C]`` (one dtype), float32 arithmetic, the sum in ascending ``r``. ``log``: the decays'
+    logarithms ``-exp(...)`` instead (what the recurrence kernels take)."""
     _dev(a, "a", F32, 2)
     _dev(w2t, "w2t", (F32, BF16), 2)
     _dev(w0, "w0", w2t.dtype, 1)
@@ -1713,7 +1733,7 @@ def channel_decay(a: torch.Tensor, col: int, w2t: torch.Tensor, w0: torch.Tensor
         raise ValueError(f"a first step of {r} outputs: the kernel takes up to {CHANNEL_DECAY_MAX_RANK}")
     out = torch.empty((a.shape[0], c), dtype=F32, device=a.device)
     _check(library().ms_channel_decay(a.data_ptr(), a.shape[1], int(col), w2t.data_ptr(), w0.data_ptr(), int(w2t.dtype == BF16),
-                                      out.data_ptr(), a.shape[0], c, r, _stream()), "channel_decay")
+                                      out.data_ptr(), a.shape[0], c, r, int(log), _stream()), "channel_decay")
     return out
 
 # ------------------------------------------------------------------------------------- sampling

@@ -254,7 +254,7 @@ class WKV(_RecurrentMixer):
         x32 = torch.empty((x.shape[0], self.ld), dtype=torch.float32, device=x.device)
         for i, (k, w) in enumerate(zip(("q", "k", "v", "g", "a"), self.weights)):
             ops.linear(blends[i], w, out=x32[:, c[k] : c[k] + w.shape[0]])
-        decay = ops.channel_decay(x32, c["a"], self.w2t, self.w0)
+        decay = ops.channel_decay(x32, c["a"], self.w2t, self.w0, log=True)
         o = ops.gated_recurrence(x32, c, self.heads, self.dim, self.dim, batch, state, mode="wkv", channel_decay=decay, bonus=self.u)
         y = ops.group_rmsnorm_gate(o, self.dim, self.norm, x32[:, c["g"] : c["g"] + n], self.eps, self.rt.dtype, "silu")
         return ops.linear(y, self.o, accumulate_into=residual, defer=True)

@@ -277,6 +277,7 @@ def test_decay_per_channel(channels, rank):
     want = np.exp(-np.exp(np.tanh(a[:, 9 : 9 + rank]) @ w2.T + w0))
     got = o.channel_decay(dev(a), 9, dev(w2.T), dev(w0))
     close(got, want, torch.float32, tol=2e-5)
+    close(o.channel_decay(dev(a), 9, dev(w2.T), dev(w0), log=True), np.log(want), torch.float32, tol=2e-5)
     wb, w0b = rounded(w2, torch.bfloat16), rounded(w0, torch.bfloat16)
     got = o.channel_decay(dev(a), 9, dev(w2.T, torch.bfloat16), dev(w0, torch.bfloat16))
     close(got, np.exp(-np.exp(np.tanh(a[:, 9 : 9 + rank]) @ wb.T + w0b)), torch.float32, tol=2e-5)
@@ -332,7 +333,7 @@ def test_recurrence_with_a_decay_per_channel_and_a_bonus(heads, dim):
                 x[off : off + c, 4 : 4 + 3 * n] = np.concatenate([r, k, v], axis=1)
                 wd[off : off + c] = w
                 off += c
-            out = o.gated_recurrence(dev(x), cols, heads, dim, dim, b, {"S": S}, mode="wkv", channel_decay=dev(wd), bonus=dev(u))
+            out = o.gated_recurrence(dev(x), cols, heads, dim, dim, b, {"S": S}, mode="wkv", channel_decay=dev(np.log(wd)), bonus=dev(u))
             off = 0
             for i, c in rows:
                 got[i].append(out[off : off + c])
