@@ -28,6 +28,26 @@ import math
 import numpy as np
 
 
+# ---------------------------------------------------------------- rounding, for error estimates
+
+
+def no_rounding(a):
+    return a
+
+
+def to_bfloat16(a):
+    """``a`` rounded to the nearest bfloat16 (ties to even), as float64: what a 16-bit product is fed."""
+    bits = np.ascontiguousarray(a, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    bits = ((bits + 0x7FFF + ((bits >> 16) & 1)) >> 16) << 16
+    return bits.astype(np.uint32).view(np.float32).astype(np.float64).reshape(np.shape(a))
+
+
+# What every matrix product's input goes through. ``forward(..., rounding=to_bfloat16)`` rounds them as a 16-bit engine
+# must (norm outputs, blends, what the output and down projections read), and nothing else: the difference to the exact
+# result is a sample of the error that rounding alone causes at each position.
+_round = no_rounding
+
+
 # ---------------------------------------------------------------- norms and activations
 
 
@@ -122,7 +142,7 @@ def attention(h, w, m, eps, positions):
         g = head // (H // G)
         s = (q[:, head] @ k[:, g].T) * m["scale"]
         out[:, head] = (softmax_over(s, seen) @ v[:, g]) * gate[:, head : head + 1]
-    return out.reshape(T, H * D) @ w["o"].T
+    return _round(out.reshape(T, H * D)) @ w["o"].T
 
 
 def retention(h, w, m, eps, positions):
@@ -141,7 +161,7 @@ def retention(h, w, m, eps, positions):
             S = float(m["decay"][head]) * S + np.outer(k[t, head], v[t, head])
             out[t, head] = S.T @ q[t, head]
     out = unit_rms(out, eps).reshape(T, H * E) * silu(h @ w["g"].T)
-    return out @ w["o"].T
+    return _round(out) @ w["o"].T
 
 
 def shifted(h):
@@ -153,7 +173,7 @@ def wkv(h, w, m, eps):
     T = h.shape[0]
     H, D = m["heads"], m["dim"]
     back = shifted(h) - h
-    mix = {s: h + back * w[f"mu.{s}"] for s in "rkvgw"}
+    mix = {s: _round(h + back * w[f"mu.{s}"]) for s in "rkvgw"}
     r = (mix["r"] @ w["r"].T).reshape(T, H, D)
     k = (mix["k"] @ w["k"].T).reshape(T, H, D)
     v = (mix["v"] @ w["v"].T).reshape(T, H, D)
@@ -167,14 +187,14 @@ def wkv(h, w, m, eps):
             out[t, head] = (S + w["u"][head][:, None] * kv).T @ r[t, head]
             S = decay[t, head][:, None] * S + kv
     out = unit_rms(out, eps).reshape(T, H * D) * w["norm"] * gate
-    return out @ w["o"].T
+    return _round(out) @ w["o"].T
 
 
 # ---------------------------------------------------------------- feed-forwards
 
 
 def dense_ff(h, w):
-    return gelu_tanh(h @ w["up"].T) @ w["down"].T
+    return _round(gelu_tanh(h @ w["up"].T)) @ w["down"].T
 
 
 def route(h, w, router):
@@ -205,7 +225,7 @@ def mixture_ff(h, w, mlp):
             if e >= router["experts"]:
                 out[t] += p * h[t]
             else:
-                out[t] += p * (relu_squared(h[t] @ w[f"e{e}.up"].T) @ w[f"e{e}.down"].T)
+                out[t] += p * (_round(relu_squared(h[t] @ w[f"e{e}.up"].T)) @ w[f"e{e}.down"].T)
     return out
 
 
@@ -216,9 +236,18 @@ def _sub(weights, prefix):
     return {k[len(prefix):]: v for k, v in weights.items() if k.startswith(prefix)}
 
 
-def forward(cfg, weights, tokens, return_layers=False, watch=None):
+def forward(cfg, weights, tokens, return_layers=False, watch=None, rounding=None):
     """Logits ``[T, vocab]`` of one sequence (and, asked for, the stream after every layer ``[layers, T, W]``).
-    ``watch(i, x)`` is shown the stream that layer ``i``'s feed-forward norm reads."""
+    ``watch(i, x)`` is shown the stream that layer ``i``'s feed-forward norm reads. ``rounding``: see ``_round``."""
+    global _round
+    before, _round = _round, rounding or no_rounding
+    try:
+        return _forward(cfg, weights, tokens, return_layers, watch)
+    finally:
+        _round = before
+
+
+def _forward(cfg, weights, tokens, return_layers, watch):
     eps = cfg["norm"]["eps"]
     tokens = np.asarray(tokens)
     positions = np.arange(len(tokens))
@@ -227,7 +256,7 @@ def forward(cfg, weights, tokens, return_layers=False, watch=None):
     for i, layer in enumerate(cfg["layers"]):
         p = f"l{layer.get('weights_of', i)}."
         w, m = _sub(weights, p + "mix."), layer["mixer"]
-        h = one_plus_norm(x, weights[p + "norm1"], eps)
+        h = _round(one_plus_norm(x, weights[p + "norm1"], eps))
         if layer["type"] == "attention":
             y = attention(h, w, m, eps, positions)
         elif layer["type"] == "retention":
@@ -242,11 +271,11 @@ def forward(cfg, weights, tokens, return_layers=False, watch=None):
             wf = _sub(weights, p + "mlp.")
             if watch is not None:
                 watch(i, x)
-            h = one_plus_norm(x, weights[p + "norm2"], eps)
+            h = _round(one_plus_norm(x, weights[p + "norm2"], eps))
             y = dense_ff(h, wf) if mlp["kind"] == "dense" else mixture_ff(h, wf, mlp)
             x = x + one_plus_norm(y, weights[p + "norm2b"], eps)
         after.append(x.copy())
-    logits = one_plus_norm(x, weights["final.norm"], eps) @ weights["embed"].T
+    logits = _round(one_plus_norm(x, weights["final.norm"], eps)) @ weights["embed"].T
     return (logits, np.stack(after)) if return_layers else logits
 
 

@@ -14,6 +14,7 @@ import torch
 
 from plain import zigelorn_plain as Z
 from plain.model_folder import read_model_folder
+from tolerances import check_logits_against_rounding
 from tolerances import check_logits_by_position as check_logits
 from zigelorn_models import ZIGELORN, make_folder, tokens_for
 
@@ -652,6 +653,75 @@ def test_the_models_show_what_is_left_out(name, folders, plain_logits):
                 assert moved(other(i, lambda l: l["mlp"]["router"].update(top=l["mlp"]["router"]["top"] - 1))) > floor, (name, i, "choices")
             if r.get("groups") and r["groups"]["keep"] < min(r["top"], r["groups"]["count"]):  # (the best k outputs lie in the best k groups)
                 assert moved(other(i, lambda l: l["mlp"]["router"].pop("groups"))) > floor, (name, i, "groups")
+
+
+def random_config(seed):
+    """A configuration drawn at random: any order of the mixers, any sizes (odd ones among them), layers that run an
+    earlier layer's weights, with and without rotation, window, groups, identity experts and feed-forward."""
+    from zigelorn_models import again, attention, dense, model, moe, retention, slowed, wkv
+
+    rng = np.random.default_rng(seed)
+    pick = lambda *a: a[int(rng.integers(0, len(a)))]
+    width = int(pick(48, 72, 100, 136, 200))
+    layers = []
+    for i in range(int(rng.integers(2, 7))):
+        if layers and rng.random() < 0.25:
+            layers.append(again(layers, int(pick(*[j for j, l in enumerate(layers) if l.get("weights_of") is None]))))
+            continue
+        outputs = int(pick(2, 4, 6, 12, 16))
+        count = int(pick(*[c for c in (1, 2, 3, 4) if outputs % c == 0]))
+        keep = int(rng.integers(1, count + 1))
+        identity = int(pick(0, 0, 1, outputs // 2))
+        top = int(rng.integers(1, min(6, outputs // count * keep) + 1))
+        mlp = pick(None, dense(int(pick(40, 96, 130))),
+                   moe(outputs - identity, top, int(pick(16, 40, 72)), identity=identity, groups=(count, keep) if count > 1 or rng.random() < 0.5 else None))
+        kind = pick("attention", "retention", "wkv")
+        if kind == "attention":
+            kv = int(pick(1, 2, 3))
+            dim = int(pick(8, 12, 20, 32, 48, 64, 80))
+            dims = int(pick(2, dim // 2 // 2 * 2, dim))
+            rot = pick(None, {"base": 200.0, "dims": dims}, slowed(1000.0, dims, float(pick(2.0, 8.0)), int(pick(16, 64)), 8.0, 1.0))
+            layers.append(attention(kv * int(pick(1, 2, 4)), kv, dim, float(pick(0.1, 0.3, dim ** -0.5)), rot, pick(None, 1, 5, 16, 33, 70), mlp))
+        elif kind == "retention":
+            heads, dim = int(pick(1, 3, 4)), int(pick(6, 16, 40, 64, 136))
+            dims = int(pick(2, dim // 2 // 2 * 2, dim))
+            decay = [float(1.0 - 2.0 ** -rng.uniform(1, 9)) for _ in range(heads)]
+            layers.append(retention(heads, dim, int(pick(8, 24, 64, 130)), decay, pick(None, {"base": 100.0, "dims": dims}), mlp))
+        else:
+            layers.append(wkv(int(pick(1, 2, 5)), int(pick(6, 16, 32, 64, 72)), int(pick(1, 7, 32)), mlp))
+    return model(int(pick(50, 131, 300)), width, float(pick(1e-6, 1e-5, 1e-3)), layers)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_configurations_drawn_at_random(seed, tmp_path):
+    """Random sizes and orders in float32, where a router's choice needs no help: whole, in portions, decoded, and two
+    requests side by side, against the plain implementation."""
+    from miniserve_amd.weights.random_init import Init, write_model_folder
+
+    cfg = random_config(seed)
+    folder = write_model_folder(tmp_path / "m", cfg, seed, Init(0.15, (0.6, 1.4)))
+    cfg, w = read_model_folder(folder)
+    rng = np.random.default_rng(seed)
+    reqs = {"a": rng.integers(0, cfg["vocab"], size=90).tolist(), "b": rng.integers(0, cfg["vocab"], size=41).tolist()}
+    want = {r: Z.forward(cfg, w, t) for r, t in reqs.items()}
+    runner = make_runner(folder, "float32", 16 * 10, 2)
+    for steps in ([[("a", 90)], [("b", 41)]], [[("a", 37), ("b", 2)], [("a", 1), ("b", 20)], [("a", 2), ("b", 1)]] + [[("a", 1), ("b", 1)]] * 18 +
+                  [[("a", 32)]]):
+        got = run_schedule(runner, reqs, steps)
+        assert runner.cache.idle
+        for r in reqs:
+            check_logits(got[r], want[r], "float32", f"seed {seed} request {r}: {[l['type'] for l in cfg['layers']]}")
+    # bfloat16 runs the same sizes through other kernels. Where no router could choose otherwise for a rounded input the
+    # logits are held to the plain implementation's, by the measure of what rounding alone does to these weights at each
+    # position (random weights of this spread make single positions several times as touchy as the rest); elsewhere they
+    # are at least numbers.
+    runner = make_runner(folder, "bfloat16", 16 * 10, 2)
+    got = run_schedule(runner, reqs, [[("a", 37), ("b", 2)], [("a", 1), ("b", 20)], [("a", 2), ("b", 1)]] + [[("a", 1), ("b", 1)]] * 18 + [[("a", 32)]])
+    routed = any((layer.get("mlp") or {}).get("kind") == "moe" for layer in cfg["layers"])
+    for r in reqs:
+        assert np.isfinite(got[r]).all()
+        if not routed:
+            check_logits_against_rounding(got[r], want[r], Z.forward(cfg, w, reqs[r], rounding=Z.to_bfloat16), f"seed {seed} request {r} in bfloat16")
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

@@ -56,3 +56,30 @@ def check_logits_by_position(got: np.ndarray, want: np.ndarray, dtype: str, what
     over = int((worst > BF16_REL_MAX * scale).sum())
     assert over <= max(1, int(BF16_FEW * len(worst))), f"{what}: bfloat16 max |diff| above {BF16_REL_MAX * scale:.3e} at {over} of {len(worst)} positions"
     assert worst.max() <= BF16_REL_CAP * scale, f"{what}: bfloat16 max |diff| {worst.max():.3e} > {BF16_REL_CAP * scale:.3e}"
+
+
+ROUNDING_TIMES = 3.0   # how many times the error that rounding alone causes a bfloat16 engine may be off at a position
+ROUNDING_WORST = 1.5   # ... and how far beyond that the worst position may lie
+
+
+def check_logits_against_rounding(got: np.ndarray, want: np.ndarray, rounded: np.ndarray, what: str = "") -> None:
+    """A bfloat16 engine against the exact logits ``want``, measured by the error that rounding alone causes: ``rounded`` are
+    the plain implementation's logits with every matrix product's input rounded to bfloat16 and nothing else changed.
+    A position's error is the root mean square over the vocabulary of the difference (its mean taken off); it may be
+    ``ROUNDING_TIMES`` the rounding sample's at that position (the sample is one draw: it is not taken below a third of
+    its own median over the positions), at all positions but 2 % (at least one), and ``ROUNDING_WORST`` times that at
+    the worst."""
+    assert got.shape == want.shape == rounded.shape, f"{what}: shapes {got.shape}, {want.shape}, {rounded.shape}"
+    assert np.isfinite(got).all(), f"{what}: non-finite logits"
+
+    def per_position(a):
+        d = a.astype(np.float64) - want
+        d = d - d.mean(axis=-1, keepdims=True)
+        return np.sqrt((d * d).mean(axis=-1))
+
+    noise = per_position(rounded)
+    limit = ROUNDING_TIMES * np.maximum(noise, np.median(noise) / 3.0)
+    ratio = per_position(got) / limit
+    over = int((ratio > 1.0).sum())
+    assert over <= max(1, int(0.02 * len(ratio))), f"{what}: {over} of {len(ratio)} positions beyond {ROUNDING_TIMES} times the rounding error (worst {ratio.max():.2f})"
+    assert ratio.max() <= ROUNDING_WORST, f"{what}: a position at {ratio.max():.2f} times its limit"
