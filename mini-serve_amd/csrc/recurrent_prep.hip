@@ -61,7 +61,8 @@ __global__ __launch_bounds__(256) void token_shift_mix_kernel(const T* __restric
   const T* hr = h + (size_t)t * W;
   const T* pr = first ? nullptr : h + (size_t)(t - 1) * W;
   const T* last = h + (size_t)(t1 - 1) * W;
-  for (int c = threadIdx.x; c < W; c += 256) {
+  const int c = blockIdx.y * 256 + threadIdx.x;  // a block per token and run of 256 channels: few tokens still make many blocks
+  if (c < W) {
     const float x = to_f32(hr[c]);
     const float p = first ? (fresh ? 0.f : cr[c]) : to_f32(pr[c]);
     const float back = p - x;
@@ -77,8 +78,10 @@ extern "C" int ms_token_shift_mix(const void* h, const void* mu, void* out, int 
   if (h == nullptr || mu == nullptr || out == nullptr || carry == nullptr || token_row == nullptr || row_start == nullptr ||
       starts == nullptr || state_slots == nullptr || W <= 0 || n <= 0)
     return MS_BAD_ARG;
-  if (is_bf16) token_shift_mix_kernel<bf16><<<tokens, 256, 0, st>>>((const bf16*)h, (const bf16*)mu, (bf16*)out, carry, token_row, row_start, starts, state_slots, tokens, W, n);
-  else token_shift_mix_kernel<float><<<tokens, 256, 0, st>>>((const float*)h, (const float*)mu, (float*)out, carry, token_row, row_start, starts, state_slots, tokens, W, n);
+  const dim3 grid(tokens, (W + 255) / 256);
+  if (grid.y > 65535) return MS_UNSUPPORTED;
+  if (is_bf16) token_shift_mix_kernel<bf16><<<grid, 256, 0, st>>>((const bf16*)h, (const bf16*)mu, (bf16*)out, carry, token_row, row_start, starts, state_slots, tokens, W, n);
+  else token_shift_mix_kernel<float><<<grid, 256, 0, st>>>((const float*)h, (const float*)mu, (float*)out, carry, token_row, row_start, starts, state_slots, tokens, W, n);
   return launch_status();
 }
 
@@ -86,7 +89,8 @@ extern "C" int ms_token_shift_mix(const void* h, const void* mu, void* out, int 
 // out[t][c] = exp(-exp(sum_r w2t[r][c] tanh(a[t][col + r]) + w0[c])), c < C, r < R: the decay of channel c at token t; or,
 // as_log, its logarithm -exp(...), which a sum over tokens keeps sharp where the decay is next to one.
 // a: float32 [tokens, lda] (the first step's projection); w2t: the second step's weight transposed, [R, C]; w0 [C].
-// Float32 throughout, the sum in ascending r. One block per token; tanh(a[t]) goes through LDS.
+// Float32 throughout, the sum in ascending r. One block per token and run of 256 channels; tanh(a[t]) goes through LDS, and
+// the weights of eight steps are asked for before they are used (a decode step is a chain of loads otherwise).
 #define DECAY_MAX_RANK 1024
 template <typename TW>
 __global__ __launch_bounds__(256) void channel_decay_kernel(const float* __restrict__ a, int lda, int col, const TW* __restrict__ w2t,
@@ -96,9 +100,17 @@ __global__ __launch_bounds__(256) void channel_decay_kernel(const float* __restr
   const int t = blockIdx.x;
   for (int r = threadIdx.x; r < R; r += 256) th[r] = tanhf(a[(size_t)t * lda + col + r]);
   __syncthreads();
-  for (int c = threadIdx.x; c < C; c += 256) {
+  const int c = blockIdx.y * 256 + threadIdx.x;
+  if (c < C) {
     float z = 0.f;
-    for (int r = 0; r < R; ++r) z = fmaf(to_f32(w2t[(size_t)r * C + c]), th[r], z);
+    for (int r0 = 0; r0 < R; r0 += 8) {
+      float w[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) w[i] = r0 + i < R ? to_f32(w2t[(size_t)(r0 + i) * C + c]) : 0.f;
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        if (r0 + i < R) z = fmaf(w[i], th[r0 + i], z);
+    }
     const float l = -expf(z + to_f32(w0[c]));
     out[(size_t)t * C + c] = as_log ? l : expf(l);
   }
@@ -109,7 +121,9 @@ extern "C" int ms_channel_decay(const float* a, int lda, int col, const void* w2
   if (tokens <= 0) return MS_OK;
   if (a == nullptr || w2t == nullptr || w0 == nullptr || out == nullptr || C <= 0 || R <= 0 || col < 0 || col + R > lda) return MS_BAD_ARG;
   if (R > DECAY_MAX_RANK) return MS_UNSUPPORTED;
-  if (w_is_bf16) channel_decay_kernel<bf16><<<tokens, 256, 0, st>>>(a, lda, col, (const bf16*)w2t, (const bf16*)w0, out, C, R, as_log);
-  else channel_decay_kernel<float><<<tokens, 256, 0, st>>>(a, lda, col, (const float*)w2t, (const float*)w0, out, C, R, as_log);
+  const dim3 grid(tokens, (C + 255) / 256);
+  if (grid.y > 65535) return MS_UNSUPPORTED;
+  if (w_is_bf16) channel_decay_kernel<bf16><<<grid, 256, 0, st>>>(a, lda, col, (const bf16*)w2t, (const bf16*)w0, out, C, R, as_log);
+  else channel_decay_kernel<float><<<grid, 256, 0, st>>>(a, lda, col, (const float*)w2t, (const float*)w0, out, C, R, as_log);
   return launch_status();
 }

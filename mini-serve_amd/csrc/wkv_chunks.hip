@@ -10,7 +10,8 @@
 //   3. per chunk, with the state S0 before it:
 //      o_t = S0^T (r_t * exp(B_t)) + sum_(j < t) P_tj v_j + (r_t . (u * k_t)) v_t,   P_tj = sum_d r_t[d] k_j[d] exp(B_t[d] - A_j[d]).
 // Every exponent is a sum of log decays and so at most zero: nothing is ever divided by a decay. All float32; sums are
-// reassociated against the token-by-token kernel (which multiplies by exp(l_t) token after token), nothing else differs.
+// reassociated against the token-by-token kernel (which multiplies by exp(l_t) token after token), nothing else differs;
+// the exponentials are the hardware's exp2 of a float32 product (an error of a unit or two in the last place).
 // The running sums are float32: where they are large the decays they stand for are next to nothing. Head sizes up to
 // WKV_CHUNK_MAX_DIM; larger ones take the token-by-token kernel.
 #include "common.h"
@@ -95,10 +96,10 @@ __global__ __launch_bounds__(256) void wkv_chunk_summary_kernel(WkvChunkArgs a) 
   __syncthreads();
   for (int i = tid; i < WKV_CHUNK * DP; i += 256) {
     const int t = i / DP, d = i % DP;
-    Kw[i] *= expf(A[d * WKV_CS + WKV_CHUNK - 1] - A[d * WKV_CS + t]);  // tokens past the count hold zero keys and zero logs
+    Kw[i] *= __expf(A[d * WKV_CS + WKV_CHUNK - 1] - A[d * WKV_CS + t]);  // tokens past the count hold zero keys and zero logs
   }
   const size_t at = (size_t)blockIdx.x * a.H + h;
-  if (tid < D) a.G[at * D + tid] = expf(A[tid * WKV_CS + WKV_CHUNK - 1]);
+  if (tid < D) a.G[at * D + tid] = __expf(A[tid * WKV_CS + WKV_CHUNK - 1]);
   __syncthreads();
   // U[d][e]: 4 x 4 outputs a thread
   const int tiles = DP / 4;
@@ -217,7 +218,7 @@ __global__ __launch_bounds__(256) void wkv_chunk_output_kernel(WkvChunkArgs a) {
           for (int j = 0; j < 4; ++j) {
             const int t = t0 + i, jj = j0 + j;
             // j < t: what is left of key j's channel when token t reads it; j == t: the bonus; j > t: nothing
-            const float wgt = jj < t ? expf(bb[i] - aa[j]) : (jj == t ? ud : 0.f);
+            const float wgt = jj < t ? __expf(bb[i] - aa[j]) : (jj == t ? ud : 0.f);
             acc[i][j] = fmaf(rr[i] * kk[j], wgt, acc[i][j]);
           }
       }
@@ -229,11 +230,20 @@ __global__ __launch_bounds__(256) void wkv_chunk_output_kernel(WkvChunkArgs a) {
   __syncthreads();
   for (int i = tid; i < DP * C; i += 256) {  // what of the state before the chunk token t still reads
     const int at = (i / C) * CS + i % C;
-    R[at] *= expf(Bx[at]);
+    R[at] *= __expf(Bx[at]);
+  }
+  __syncthreads();
+  // The state before the chunk takes the keys' place in LDS: [D][DP], zero beyond D.
+  {
+    const float* S0g = a.U + ((size_t)blockIdx.x * a.H + h) * (size_t)D * D;
+    for (int i = tid; i < D * DP; i += 256) {
+      const int d = i / DP, e = i % DP;
+      K[i] = e < D ? S0g[(size_t)d * D + e] : 0.f;
+    }
   }
   __syncthreads();
   // o[t][e]: 4 x 4 outputs a thread
-  const float* S0 = a.U + ((size_t)blockIdx.x * a.H + h) * (size_t)D * D;
+  const float* S0 = K;
   const int etiles = DP / 4;
   for (int tile = tid; tile < (C / 4) * etiles; tile += 256) {
     const int t0 = (tile / etiles) * 4, e0 = (tile % etiles) * 4;
@@ -242,9 +252,8 @@ __global__ __launch_bounds__(256) void wkv_chunk_output_kernel(WkvChunkArgs a) {
     for (int d = 0; d < D; ++d) {
       const float4 r4 = *reinterpret_cast<const float4*>(R + d * CS + t0);
       const float rr[4] = {r4.x, r4.y, r4.z, r4.w};
-      float sv[4];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) sv[j] = e0 + j < D ? S0[(size_t)d * D + e0 + j] : 0.f;
+      const float4 s4 = *reinterpret_cast<const float4*>(S0 + d * DP + e0);
+      const float sv[4] = {s4.x, s4.y, s4.z, s4.w};
 #pragma unroll
       for (int i = 0; i < 4; ++i)
 #pragma unroll
