@@ -90,9 +90,14 @@ __device__ __forceinline__ float sum_splits(const float* __restrict__ p, int spl
 #define MS_GATED_COUNT 3
 // The square of max(x, 0): only as the activation of a feed-forward without a gate.
 #define MS_ACT_RELU_SQUARED 3
-static __host__ __device__ __forceinline__ bool ms_act_ungated_ok(int act) { return act == MS_ACT_SILU || act == MS_ACT_GELU_TANH || act == MS_ACT_RELU_SQUARED; }
+// The hyperbolic tangent: between the two steps of a small projection, never in a feed-forward's gate.
+#define MS_ACT_TANH 4
+static __host__ __device__ __forceinline__ bool ms_act_ungated_ok(int act) {
+  return act == MS_ACT_SILU || act == MS_ACT_GELU_TANH || act == MS_ACT_RELU_SQUARED || act == MS_ACT_TANH;
+}
 __device__ __forceinline__ float activate(float x, int act) {
   if (act == MS_ACT_RELU_SQUARED) { const float r = fmaxf(x, 0.f); return r * r; }
+  if (act == MS_ACT_TANH) return tanhf(x);
   if (act == MS_ACT_GELU_TANH) return 0.5f * x * (1.f + tanhf(0.7978845608028654f * (x + 0.044715f * x * x * x)));
   return x / (1.f + expf(-x));
 }

@@ -1,7 +1,7 @@
 // What recurrent mixers do to their projections before the recurrence runs, all in float32:
 //   * a rotation of the query and key heads of a float32 projection, in place, with a scale on the way;
 //   * the blends of a token's input with the previous token's, one per projection, and the carry of the last input;
-//   * a decay per channel and token out of a small two-step projection.
+//   * the last step of a decay per channel and token out of a small two-step projection.
 #include "common.h"
 
 // ---------------------------------------------------------------------------------------------
@@ -86,44 +86,24 @@ extern "C" int ms_token_shift_mix(const void* h, const void* mu, void* out, int 
 }
 
 // ---------------------------------------------------------------------------------------------
-// out[t][c] = exp(-exp(sum_r w2t[r][c] tanh(a[t][col + r]) + w0[c])), c < C, r < R: the decay of channel c at token t; or,
-// as_log, its logarithm -exp(...), which a sum over tokens keeps sharp where the decay is next to one.
-// a: float32 [tokens, lda] (the first step's projection); w2t: the second step's weight transposed, [R, C]; w0 [C].
-// Float32 throughout, the sum in ascending r. One block per token and run of 256 channels; tanh(a[t]) goes through LDS, and
-// the weights of eight steps are asked for before they are used (a decode step is a chain of loads otherwise).
-#define DECAY_MAX_RANK 1024
-template <typename TW>
-__global__ __launch_bounds__(256) void channel_decay_kernel(const float* __restrict__ a, int lda, int col, const TW* __restrict__ w2t,
-                                                            const TW* __restrict__ w0, float* __restrict__ out, int C, int R,
-                                                            int as_log) {
-  __shared__ float th[DECAY_MAX_RANK];
-  const int t = blockIdx.x;
-  for (int r = threadIdx.x; r < R; r += 256) th[r] = tanhf(a[(size_t)t * lda + col + r]);
-  __syncthreads();
-  const int c = blockIdx.y * 256 + threadIdx.x;
-  if (c < C) {
-    float z = 0.f;
-    for (int r0 = 0; r0 < R; r0 += 8) {
-      float w[8];
-#pragma unroll
-      for (int i = 0; i < 8; ++i) w[i] = r0 + i < R ? to_f32(w2t[(size_t)(r0 + i) * C + c]) : 0.f;
-#pragma unroll
-      for (int i = 0; i < 8; ++i)
-        if (r0 + i < R) z = fmaf(w[i], th[r0 + i], z);
-    }
-    const float l = -expf(z + to_f32(w0[c]));
-    out[(size_t)t * C + c] = as_log ? l : expf(l);
-  }
+// z[t][c] <- -exp(z[t][c] + b[c]), or, as_decay, exp of that: the last step of a decay per channel and token,
+// w = exp(-exp(W2 tanh(W1 x) + w0)). The two products and the tanh between them are the engine's float32 product and
+// activation kernels; the logarithm -exp(...) is what the recurrence kernels take (a sum over tokens keeps it sharp where
+// the decay is next to one). Float32, in place.
+template <typename TB>
+__global__ void neg_exp_bias_kernel(float* __restrict__ z, const TB* __restrict__ b, size_t n, int C, int as_decay) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const float l = -expf(z[i] + to_f32(b[i % C]));
+  z[i] = as_decay ? expf(l) : l;
 }
 
-extern "C" int ms_channel_decay(const float* a, int lda, int col, const void* w2t, const void* w0, int w_is_bf16, float* out,
-                                int tokens, int C, int R, int as_log, hipStream_t st) {
+extern "C" int ms_neg_exp_bias(float* z, const void* b, int b_is_bf16, int tokens, int C, int as_decay, hipStream_t st) {
   if (tokens <= 0) return MS_OK;
-  if (a == nullptr || w2t == nullptr || w0 == nullptr || out == nullptr || C <= 0 || R <= 0 || col < 0 || col + R > lda) return MS_BAD_ARG;
-  if (R > DECAY_MAX_RANK) return MS_UNSUPPORTED;
-  const dim3 grid(tokens, (C + 255) / 256);
-  if (grid.y > 65535) return MS_UNSUPPORTED;
-  if (w_is_bf16) channel_decay_kernel<bf16><<<grid, 256, 0, st>>>(a, lda, col, (const bf16*)w2t, (const bf16*)w0, out, C, R, as_log);
-  else channel_decay_kernel<float><<<grid, 256, 0, st>>>(a, lda, col, (const float*)w2t, (const float*)w0, out, C, R, as_log);
+  if (z == nullptr || b == nullptr || C <= 0) return MS_BAD_ARG;
+  const size_t n = (size_t)tokens * C;
+  const unsigned blocks = (unsigned)((n + 255) / 256);
+  if (b_is_bf16) neg_exp_bias_kernel<bf16><<<blocks, 256, 0, st>>>(z, (const bf16*)b, n, C, as_decay);
+  else neg_exp_bias_kernel<float><<<blocks, 256, 0, st>>>(z, (const float*)b, n, C, as_decay);
   return launch_status();
 }

@@ -39,7 +39,7 @@ _SIGNATURES = {
                             _c_int, _c_void, _c_int, _c_void, _c_void],
     "ms_rotate_columns": [_c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void, _c_int, _c_int, _c_float, _c_void],
     "ms_token_shift_mix": [_c_void, _c_void, _c_void, _c_int, _c_void, _c_void, _c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_void],
-    "ms_channel_decay": [_c_void, _c_int, _c_int, _c_void, _c_void, _c_int, _c_void, _c_int, _c_int, _c_int, _c_int, _c_void],
+    "ms_neg_exp_bias": [_c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_void],
     "ms_wkv_chunked": [_c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void, _c_int, _c_void, _c_void, _c_void, _c_void, _c_void,
                        _c_void, _c_int, _c_int, _c_void, _c_void, _c_void],
     "ms_wkv_chunk_tokens": [],
@@ -302,8 +302,8 @@ def interleave_gate_up(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
 # silu(x) = x sigmoid(x); gelu_tanh(x) = x / 2 (1 + tanh(sqrt(2 / pi) (x + 0.044715 x^3))).
 # swiglu_clamped(gate, up) = g sigmoid(1.702 g) (u + 1) with g = min(gate, limit), u = clamp(up, -limit, limit): not of
 # the form act(gate) * up, it takes ``limit`` along and runs in the activation kernels (no matrix kernel's epilogue knows it).
-ACTIVATIONS = {"silu": 0, "gelu_tanh": 1, "swiglu_clamped": 2, "relu_squared": 3}
-ACTIVATIONS_UNGATED_ONLY = {"relu_squared"}  # no kernel finishes act(gate) * up with these
+ACTIVATIONS = {"silu": 0, "gelu_tanh": 1, "swiglu_clamped": 2, "relu_squared": 3, "tanh": 4}
+ACTIVATIONS_UNGATED_ONLY = {"relu_squared", "tanh"}  # no kernel finishes act(gate) * up with these
 ACTIVATIONS_WITH_LIMIT = {"swiglu_clamped"}
 
 
@@ -1716,25 +1716,19 @@ def token_shift_mix(h: torch.Tensor, mu: torch.Tensor, carry: torch.Tensor, batc
     return out
 
 
-CHANNEL_DECAY_MAX_RANK = 1024  # DECAY_MAX_RANK in csrc/recurrent_prep.hip
-
-
-def channel_decay(a: torch.Tensor, col: int, w2t: torch.Tensor, w0: torch.Tensor, log: bool = False) -> torch.Tensor:
-    """``exp(-exp(tanh(a[:, col : col + R]) @ w2t + w0))``: float32 ``[T, C]`` from the float32 ``a [T, >= col + R]``,
-    ``w2t [R, C]`` and ``w0 [C]`` (one dtype), float32 arithmetic, the sum in ascending ``r``. ``log``: the decays'
-    logarithms ``-exp(...)`` instead (what the recurrence kernels take)."""
+def channel_decay(a: torch.Tensor, w2: torch.Tensor, w0: torch.Tensor, log: bool = False) -> torch.Tensor:
+    """``exp(-exp(tanh(a) @ w2^T + w0))``: float32 ``[T, C]`` from the float32 ``a [T, R]``, ``w2 [C, R]`` (float32: the product
+    is the true 32-bit one, a chain of multiply-adds in ascending ``r``) and ``w0 [C]``. ``log``: the decays' logarithms
+    ``-exp(...)`` instead (what the recurrence kernels take). Three launches: the tanh, the product, the exponentials."""
     _dev(a, "a", F32, 2)
-    _dev(w2t, "w2t", (F32, BF16), 2)
-    _dev(w0, "w0", w2t.dtype, 1)
-    r, c = w2t.shape
-    if col < 0 or col + r > a.shape[1] or w0.shape[0] != c:
-        raise ValueError(f"columns {col} .. {col + r} of a matrix of width {a.shape[1]}, w0 of {w0.shape[0]} for {c} channels")
-    if r > CHANNEL_DECAY_MAX_RANK:
-        raise ValueError(f"a first step of {r} outputs: the kernel takes up to {CHANNEL_DECAY_MAX_RANK}")
-    out = torch.empty((a.shape[0], c), dtype=F32, device=a.device)
-    _check(library().ms_channel_decay(a.data_ptr(), a.shape[1], int(col), w2t.data_ptr(), w0.data_ptr(), int(w2t.dtype == BF16),
-                                      out.data_ptr(), a.shape[0], c, r, int(log), _stream()), "channel_decay")
-    return out
+    _dev(w2, "w2", F32, 2)
+    _dev(w0, "w0", (F32, BF16), 1)
+    c, r = w2.shape
+    if a.shape[1] != r or w0.shape[0] != c:
+        raise ValueError(f"a {tuple(a.shape)}, w2 {tuple(w2.shape)} and w0 {tuple(w0.shape)} do not fit")
+    z = linear(activate(a, "tanh", F32), w2, out_dtype=F32)
+    _check(library().ms_neg_exp_bias(z.data_ptr(), w0.data_ptr(), int(w0.dtype == BF16), z.shape[0], c, int(not log), _stream()), "neg_exp_bias")
+    return z
 
 # ------------------------------------------------------------------------------------- sampling
 

@@ -204,7 +204,7 @@ class WKV(_RecurrentMixer):
         # the width of the decay's first step: a configuration may state it; else the checkpoint's tensors say it
         self.rank = int(spec["decay_rank"]) if spec.get("decay_rank") else None
         self.ld = 0
-        self.mu = self.weights = self.w2t = self.w0 = self.u = None
+        self.mu = self.weights = self.w2 = self.w0 = self.u = None
 
     @classmethod
     def tensors(cls, spec: PartSpec) -> dict[str, TensorSpec]:
@@ -229,17 +229,15 @@ class WKV(_RecurrentMixer):
         self.rank = self.weights[4].shape[0]
         if tensors[n["w2"]].shape[1] != self.rank:
             raise ValueError(f"{n['w1']} has {self.rank} rows, {n['w2']} {tensors[n['w2']].shape[1]} columns")
-        if not 1 <= self.rank <= self.rt.ops.CHANNEL_DECAY_MAX_RANK:
-            raise ValueError(f"{n['w1']}: {self.rank} rows; the decay's kernel takes 1..{self.rt.ops.CHANNEL_DECAY_MAX_RANK}")
         at = 0
         width = self.heads * self.dim
-        for k, cols in (("q", width), ("k", width), ("v", width), ("g", width), ("a", self.rank)):  # q: the receptance; a: the decay's first step
+        for k, cols in (("q", width), ("k", width), ("v", width), ("g", width)):  # q: the receptance
             self.columns[k] = at
             at += -(-cols // 4) * 4  # every product's columns start 16-byte aligned
         self.ld = at
         self.mu = torch.stack([tensors[n[f"mu_{k}"]].to(dtype) for k in self.BLENDS]).contiguous()
-        self.w2t = tensors[n["w2"]].t().contiguous()  # [rank, channels]: a thread per channel reads side by side
-        self.w0 = tensors[n["w0"]].to(self.w2t.dtype).contiguous()
+        self.w2 = tensors[n["w2"]].to(torch.float32).contiguous()  # the decay's second step is a true 32-bit product (widening is exact)
+        self.w0 = tensors[n["w0"]]
         self.u = tensors[n["u"]].to(torch.float32).contiguous()
         self.o, self.norm = tensors[n["o"]], tensors[n["norm"]]
 
@@ -252,15 +250,15 @@ class WKV(_RecurrentMixer):
         c, n = self.columns, self.heads * self.dim
         blends = ops.token_shift_mix(ops.cast(x, self.mu.dtype), self.mu, state["shift"], batch)
         x32 = torch.empty((x.shape[0], self.ld), dtype=torch.float32, device=x.device)
-        for i, (k, w) in enumerate(zip(("q", "k", "v", "g", "a"), self.weights)):
+        for i, (k, w) in enumerate(zip(("q", "k", "v", "g"), self.weights)):
             ops.linear(blends[i], w, out=x32[:, c[k] : c[k] + w.shape[0]])
-        decay = ops.channel_decay(x32, c["a"], self.w2t, self.w0, log=True)
+        decay = ops.channel_decay(ops.linear(blends[4], self.weights[4], out_dtype=torch.float32), self.w2, self.w0, log=True)
         o = ops.gated_recurrence(x32, c, self.heads, self.dim, self.dim, batch, state, mode="wkv", channel_decay=decay, bonus=self.u)
         y = ops.group_rmsnorm_gate(o, self.dim, self.norm, x32[:, c["g"] : c["g"] + n], self.eps, self.rt.dtype, "silu")
         return ops.linear(y, self.o, accumulate_into=residual, defer=True)
 
     def parameters_bytes(self) -> int:
-        ts = self.weights + [self.mu, self.w2t, self.w0, self.u, self.o, self.norm]
+        ts = self.weights + [self.mu, self.w2, self.w0, self.u, self.o, self.norm]
         return sum(t.numel() * t.element_size() for t in ts)
 
     def flops(self, rows) -> int:

@@ -272,16 +272,14 @@ def test_blends_with_the_previous_token_and_the_carried_row(dtype):
 def test_decay_per_channel(channels, rank):
     o = ops()
     rng = np.random.default_rng(channels)
-    T = 21
-    a = rng.normal(size=(T, 9 + rank + 3))
-    w2, w0 = rng.normal(size=(channels, rank)) / np.sqrt(rank), rng.normal(size=channels) - 1.0
-    want = np.exp(-np.exp(np.tanh(a[:, 9 : 9 + rank]) @ w2.T + w0))
-    got = o.channel_decay(dev(a), 9, dev(w2.T), dev(w0))
-    close(got, want, torch.float32, tol=2e-5)
-    close(o.channel_decay(dev(a), 9, dev(w2.T), dev(w0), log=True), np.log(want), torch.float32, tol=2e-5)
-    wb, w0b = rounded(w2, torch.bfloat16), rounded(w0, torch.bfloat16)
-    got = o.channel_decay(dev(a), 9, dev(w2.T, torch.bfloat16), dev(w0, torch.bfloat16))
-    close(got, np.exp(-np.exp(np.tanh(a[:, 9 : 9 + rank]) @ wb.T + w0b)), torch.float32, tol=2e-5)
+    for T in (1, 8, 21, 300):
+        a = rng.normal(size=(T, rank))
+        w2, w0 = rng.normal(size=(channels, rank)) / np.sqrt(rank), rng.normal(size=channels) - 1.0
+        want = np.exp(-np.exp(np.tanh(a) @ w2.T + w0))
+        close(o.channel_decay(dev(a), dev(w2), dev(w0)), want, torch.float32, tol=2e-5)
+        close(o.channel_decay(dev(a), dev(w2), dev(w0), log=True), np.log(want), torch.float32, tol=2e-5)
+        w0b = rounded(w0, torch.bfloat16)
+        close(o.channel_decay(dev(a), dev(w2), dev(w0, torch.bfloat16)), np.exp(-np.exp(np.tanh(a) @ w2.T + w0b)), torch.float32, tol=2e-5)
 
 
 def plain_wkv(r, k, v, w, u):
