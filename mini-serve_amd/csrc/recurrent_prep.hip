@@ -47,7 +47,7 @@ extern "C" int ms_rotate_columns(float* x, int ld, int col, int tokens, int H, i
 // the first token of its request's rows, else the request's carried row carry[slot] (zeros when the request starts in this
 // step). Float32 arithmetic, rounded once. The thread that reads carry[slot][c] for a request's first token is the one that
 // then writes the request's last row of this step there: one reader and one writer per element, the same thread.
-template <typename T>
+template <typename T, int VEC>
 __global__ __launch_bounds__(256) void token_shift_mix_kernel(const T* __restrict__ h, const T* __restrict__ mu, T* __restrict__ out,
                                                               float* __restrict__ carry, const int* __restrict__ token_row,
                                                               const int* __restrict__ row_start, const int* __restrict__ starts,
@@ -61,14 +61,32 @@ __global__ __launch_bounds__(256) void token_shift_mix_kernel(const T* __restric
   const T* hr = h + (size_t)t * W;
   const T* pr = first ? nullptr : h + (size_t)(t - 1) * W;
   const T* last = h + (size_t)(t1 - 1) * W;
-  const int c = blockIdx.y * 256 + threadIdx.x;  // a block per token and run of 256 channels: few tokens still make many blocks
-  if (c < W) {
-    const float x = to_f32(hr[c]);
-    const float p = first ? (fresh ? 0.f : cr[c]) : to_f32(pr[c]);
-    const float back = p - x;
-    for (int s = 0; s < n; ++s) out[((size_t)s * tokens + t) * W + c] = from_f32<T>(x + back * to_f32(mu[(size_t)s * W + c]));
-    if (first) cr[c] = to_f32(last[c]);
+  // a block per token and run of 256 VEC channels (few tokens still make many blocks); a thread owns VEC consecutive
+  // channels, 16 bytes of a row (VEC = 1: any width)
+  const int c0 = (blockIdx.y * 256 + threadIdx.x) * VEC;
+  if (c0 >= W) return;
+  struct alignas(sizeof(T) * VEC) Pack { T e[VEC]; };
+  const Pack xs = *reinterpret_cast<const Pack*>(hr + c0);
+  Pack ps, ls;
+  if (!first) ps = *reinterpret_cast<const Pack*>(pr + c0);
+  if (first) ls = *reinterpret_cast<const Pack*>(last + c0);
+  float x[VEC], back[VEC];
+#pragma unroll
+  for (int i = 0; i < VEC; ++i) {
+    x[i] = to_f32(xs.e[i]);
+    const float p = first ? (fresh ? 0.f : cr[c0 + i]) : to_f32(ps.e[i]);
+    back[i] = p - x[i];
   }
+  for (int s = 0; s < n; ++s) {
+    const Pack ms = *reinterpret_cast<const Pack*>(mu + (size_t)s * W + c0);
+    Pack o;
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) o.e[i] = from_f32<T>(x[i] + back[i] * to_f32(ms.e[i]));
+    *reinterpret_cast<Pack*>(out + ((size_t)s * tokens + t) * W + c0) = o;
+  }
+  if (first)
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) cr[c0 + i] = to_f32(ls.e[i]);
 }
 
 extern "C" int ms_token_shift_mix(const void* h, const void* mu, void* out, int is_bf16, float* carry, const int* token_row,
@@ -78,10 +96,15 @@ extern "C" int ms_token_shift_mix(const void* h, const void* mu, void* out, int 
   if (h == nullptr || mu == nullptr || out == nullptr || carry == nullptr || token_row == nullptr || row_start == nullptr ||
       starts == nullptr || state_slots == nullptr || W <= 0 || n <= 0)
     return MS_BAD_ARG;
-  const dim3 grid(tokens, (W + 255) / 256);
+  const int vec = is_bf16 ? 8 : 4;
+  const bool wide = W % vec == 0 && (size_t)h % 16 == 0 && (size_t)mu % 16 == 0 && (size_t)out % 16 == 0;
+  const int per = wide ? vec : 1;
+  const dim3 grid(tokens, (W + 256 * per - 1) / (256 * per));
   if (grid.y > 65535) return MS_UNSUPPORTED;
-  if (is_bf16) token_shift_mix_kernel<bf16><<<grid, 256, 0, st>>>((const bf16*)h, (const bf16*)mu, (bf16*)out, carry, token_row, row_start, starts, state_slots, tokens, W, n);
-  else token_shift_mix_kernel<float><<<grid, 256, 0, st>>>((const float*)h, (const float*)mu, (float*)out, carry, token_row, row_start, starts, state_slots, tokens, W, n);
+#define TSM(T, V) token_shift_mix_kernel<T, V><<<grid, 256, 0, st>>>((const T*)h, (const T*)mu, (T*)out, carry, token_row, row_start, starts, state_slots, tokens, W, n)
+  if (is_bf16) { if (wide) TSM(bf16, 8); else TSM(bf16, 1); }
+  else { if (wide) TSM(float, 4); else TSM(float, 1); }
+#undef TSM
   return launch_status();
 }
 
