@@ -4,7 +4,8 @@ architecture.
 ``config.json``: ``architecture`` (the name), ``vocab``, ``width``, ``norm.eps`` and ``layers``, a list in which every
 entry names its mixer (``type``), the mixer's sizes and constants (``mixer``) and its feed-forward (``mlp``, or null for
 none). Layer ``i``'s tensors start with ``l<i>.``. An entry with ``weights_of: j`` has no tensors: it runs layer ``j``'s
-weights (mixer, feed-forward and norms) over a cache and state of its own, and the rest of its entry equals layer ``j``'s.
+weights (mixer, feed-forward and norms) over a cache and state of its own, and the rest of its entry equals layer ``j``'s
+(``j`` may come before or after it; where ``j`` runs another layer's weights in turn, that layer's are meant).
 
 A layer is ``x += N1b(mixer(N1(x)))``, then ``x += N2b(ff(N2(x)))``, every ``N`` an RMS norm whose stored weight lies
 around zero (``y / rms(y) * (1 + w)``; tensors ``norm1 norm1b norm2 norm2b``). The mixers:
@@ -136,15 +137,10 @@ class ZigelornConfig:
                 _positive_int(m, "rank", mw)
             if kind != "wkv" and m.get("rot"):
                 _check_rot(m["rot"], m["dim"], f"{mw}.rot")
-            src = layer.get("weights_of")
-            if src is not None:
-                if not isinstance(src, int) or isinstance(src, bool) or not 0 <= src < i:
-                    raise ValueError(f"{where}.weights_of must name an earlier layer, got {src!r}")
-                if self.layers[src].get("weights_of") is not None:
-                    raise ValueError(f"{where}.weights_of names layer {src}, which has no tensors of its own")
-                other = self.layers[src]
-                if (other["type"], other["mixer"], other.get("mlp")) != (kind, m, layer.get("mlp")):
-                    raise ValueError(f"{where} runs layer {src}'s weights but its entry differs from that layer's")
+            if layer.get("weights_of") is not None:
+                root = self.source(i)
+                if self.layers[root]["type"] != kind:
+                    raise ValueError(f"{where} is a {kind!r} layer but runs the weights of layer {root}, a {self.layers[root]['type']!r} layer")
             mlp = layer.get("mlp")
             if mlp:
                 fw = f"{where}.mlp"
@@ -176,6 +172,19 @@ class ZigelornConfig:
                         choosable = outputs // count * keep
                     if top > choosable:
                         raise ValueError(f"{fw}.router: top {top} of {choosable} outputs that can be chosen")
+
+    def source(self, i: int) -> int:
+        """The layer whose tensors layer ``i`` runs: itself, or what its ``weights_of`` leads to."""
+        seen = {i}
+        while self.layers[i].get("weights_of") is not None:
+            j = self.layers[i]["weights_of"]
+            if not isinstance(j, int) or isinstance(j, bool) or not 0 <= j < len(self.layers):
+                raise ValueError(f"layers[{i}].weights_of must be the number of a layer, got {j!r}")
+            if j in seen:
+                raise ValueError(f"layers[{i}].weights_of leads back to layer {j}: no layer of the chain has tensors")
+            seen.add(j)
+            i = j
+        return i
 
     def to_dict(self) -> dict:
         """The ``config.json`` that reads back as this configuration."""
@@ -231,11 +240,9 @@ class ZigelornConfig:
 
     def to_spec(self) -> ModelSpec:
         w = self.width
-        layers, order, index = [], [], {}
+        layers, index = [], {}
         for i, layer in enumerate(self.layers):
-            src = layer.get("weights_of")
-            if src is not None:
-                order.append(RunEntry(index[src], i))  # another layer's weights over a cache and state of its own
+            if layer.get("weights_of") is not None:
                 continue
             mlp = layer.get("mlp")
             block = PartSpec("sandwich", {
@@ -244,7 +251,8 @@ class ZigelornConfig:
                 "spare": None if mlp else {"norm2": w, "norm2b": w}})
             index[i] = len(layers)
             layers.append(LayerSpec(f"l{i}.", block, self._mixer(layer["type"], layer["mixer"]), self._feed_forward(mlp)))
-            order.append(RunEntry(index[i], i))
+        # every entry runs over a cache and state of its own, whosever weights it runs
+        order = [RunEntry(index[self.source(i)], i) for i in range(len(self.layers))]
         return ModelSpec(
             architecture=self.architecture,
             vocab_size=self.vocab,

@@ -232,6 +232,13 @@ def mixture_ff(h, w, mlp):
 # ---------------------------------------------------------------- the model
 
 
+def weights_layer(cfg, i):
+    """The layer whose tensors layer ``i`` runs: itself, or the end of its chain of ``weights_of``."""
+    while cfg["layers"][i].get("weights_of") is not None:
+        i = cfg["layers"][i]["weights_of"]
+    return i
+
+
 def _sub(weights, prefix):
     return {k[len(prefix):]: v for k, v in weights.items() if k.startswith(prefix)}
 
@@ -254,7 +261,7 @@ def _forward(cfg, weights, tokens, return_layers, watch):
     x = weights["embed"][tokens].astype(np.float64)
     after = []
     for i, layer in enumerate(cfg["layers"]):
-        p = f"l{layer.get('weights_of', i)}."
+        p = f"l{weights_layer(cfg, i)}."
         w, m = _sub(weights, p + "mix."), layer["mixer"]
         h = _round(one_plus_norm(x, weights[p + "norm1"], eps))
         if layer["type"] == "attention":

@@ -76,6 +76,18 @@ def test_a_layer_that_runs_anothers_weights_has_a_state_of_its_own():
     assert [layer.prefix for layer in spec.layers] == ["l0.", "l1.", "l2.", "l5."]
 
 
+def test_weights_of_a_later_layer_and_through_another():
+    """The layer that has the tensors may come later, and may be named through a layer that runs its weights too."""
+    cfg = copy.deepcopy(ZIGELORN["zgC"][0])  # wkv, retention, wkv (weights of 0)
+    first = cfg["layers"][0]
+    cfg["layers"] = [dict(copy.deepcopy(first), weights_of=3), cfg["layers"][1], dict(copy.deepcopy(first), weights_of=0), first]
+    spec = config_from_dict(cfg).to_spec()
+    assert [layer.prefix for layer in spec.layers] == ["l1.", "l3."]
+    assert [(e.layer, e.cache) for e in spec.run_order] == [(1, 0), (0, 1), (1, 2), (1, 3)]
+    names = expected_tensors(spec)
+    assert "l3.mix.r" in names and not any(k.startswith(("l0.", "l2.")) for k in names)
+
+
 def test_cache_groups_and_states():
     """Windowed attention layers of one shape share a group; every recurrent layer keeps a state and no pages; a model
     of recurrences alone has no group at all."""
@@ -117,9 +129,10 @@ def test_config_refusals():
         (lambda c: c["layers"][1]["mixer"]["rot"].update(dims=18), ValueError),
         (lambda c: c["layers"][2]["mixer"].update(decay=[0.9]), ValueError),       # one decay per head
         (lambda c: c["layers"][2]["mixer"].update(decay=[0.9, 1.5]), ValueError),
-        (lambda c: c["layers"][3].update(weights_of=4), ValueError),               # only earlier layers
-        (lambda c: c["layers"][4].update(weights_of=3), ValueError),               # ... that have tensors of their own
-        (lambda c: c["layers"][3]["mixer"].update(heads=2), ValueError),           # ... and the same entry
+        (lambda c: c["layers"][3].update(weights_of=9), ValueError),               # no such layer
+        (lambda c: c["layers"][3].update(weights_of=3), ValueError),               # itself
+        (lambda c: c["layers"][1].update(weights_of=3), ValueError),               # a ring: nobody has the tensors
+        (lambda c: c["layers"][3].update(weights_of=0), ValueError),               # a layer of another kind
         (lambda c: c["layers"][1]["mlp"]["router"].update(top=5), ValueError),     # more than the kept groups hold
         (lambda c: c["layers"][1]["mlp"]["router"]["groups"].update(count=3), ValueError),
         (lambda c: c["layers"][1]["mlp"].update(kind="gated"), NotImplementedError),
