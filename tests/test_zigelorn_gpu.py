@@ -722,6 +722,25 @@ def test_configurations_drawn_at_random(seed, tmp_path):
             check_logits_against_rounding(got[r], want[r], Z.forward(cfg, w, reqs[r], rounding=Z.to_bfloat16), f"seed {seed} request {r} in bfloat16")
 
 
+def test_weights_of_a_later_layer_and_through_another(tmp_path):
+    """The first layer runs the last layer's weights, the third runs the first's (and so the last's): three states, one
+    set of tensors."""
+    import copy
+
+    from miniserve_amd.weights.random_init import Init, write_model_folder
+
+    cfg = copy.deepcopy(ZIGELORN["zgC"][0])
+    first = cfg["layers"][0]
+    cfg["layers"] = [dict(copy.deepcopy(first), weights_of=3), cfg["layers"][1], dict(copy.deepcopy(first), weights_of=0), first]
+    folder = write_model_folder(tmp_path / "m", cfg, 3, Init(0.15, (0.6, 1.4)))
+    cfg, w = read_model_folder(folder)
+    assert not any(k.startswith(("l0.", "l2.")) for k in w)
+    toks = np.random.default_rng(0).integers(0, cfg["vocab"], size=70).tolist()
+    runner = make_runner(folder, "float32", 128, 1)
+    got = run_schedule(runner, {"a": toks}, [[("a", n)] for n in portions(70, [20, 1, 1, 2, 30])])["a"]
+    check_logits(got, Z.forward(cfg, w, toks), "float32", "weights of a later layer")
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", sorted(ZIGELORN))
 def test_unequal_requests_in_one_batch_with_pages_and_slots_used_again(name, dtype, folders, plain_logits):
