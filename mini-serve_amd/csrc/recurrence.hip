@@ -164,9 +164,10 @@ extern "C" int ms_gated_recurrence(const float* x, int ld, int q_off, int k_off,
                                    const float* u, hipStream_t st) {
   if (rows <= 0) return MS_OK;
   if (H <= 0 || D <= 0 || E <= 0 || x == nullptr || S == nullptr || out == nullptr || row_start == nullptr || starts == nullptr ||
-      state_slots == nullptr || (act != 0 && act != 1) || q_off < 0 || k_off < 0 || v_off < 0 || q_off + H * D > ld ||
-      k_off + H * D > ld || v_off + H * E > ld)
+      state_slots == nullptr || (act != 0 && act != 1) || q_off < 0 || k_off < 0 || v_off < 0)
     return MS_BAD_ARG;
+  // (q, k and v may lie in later rows of the matrix that x is the top of: their columns are then counted past ld, and the
+  // caller answers for the rows being there)
   if (mode == MS_REC_DECAY) {
     if (decay == nullptr) return MS_BAD_ARG;
   } else if (mode == MS_REC_EXP_GATES) {

@@ -1560,7 +1560,8 @@ WKV_CHUNKED_FROM = 16  # ... and from which the recurrence with a decay per chan
 def gated_recurrence(x: torch.Tensor, columns: dict, heads: int, dim: int, value_dim: int, batch, state: dict, *,
                      mode: str, activation: str | None = None, q_scale: float = 1.0, decay: torch.Tensor | None = None,
                      cap: float = 0.0, i_bias: torch.Tensor | None = None, f_bias: torch.Tensor | None = None,
-                     chunks: bool = True, channel_decay: torch.Tensor | None = None, bonus: torch.Tensor | None = None) -> torch.Tensor:
+                     chunks: bool = True, channel_decay: torch.Tensor | None = None, bonus: torch.Tensor | None = None,
+                     rows_below: int = 0) -> torch.Tensor:
     """A linear recurrence over a matrix state per (request, head): ``S_t = a_t S_(t-1) + b_t k_t v_t^T``,
     ``o_t = S_t^T q_t``, for the step's rows (``batch.row_start``, ``batch.starts``, ``batch.state_slots``), in float32.
 
@@ -1575,6 +1576,11 @@ def gated_recurrence(x: torch.Tensor, columns: dict, heads: int, dim: int, value
     (``dim == value_dim``). Rows of ``WKV_CHUNKED_FROM`` tokens or more run in chunks (head sizes up to 64).
     ``state["S"]``: float32 ``[slots, heads, dim, value_dim]``; rows with ``starts == 0`` begin from zero.
     Returns float32 ``[T, heads * value_dim]``.
+
+    ``rows_below``: ``x`` is the top ``T`` rows of a matrix that has so many rows more (one product of stacked inputs against
+    stacked weights leaves each projection in a block of rows of its own); a column number may then count on past the row's
+    end into those rows (column ``j * T * ld + c`` is column ``c`` of the row ``j T`` rows further down). Token-by-token
+    kernel only.
 
     Two kernel families compute the same thing: one walks a row's tokens in order with the state in registers (decode
     steps, short portions, head sizes above 128); the other works in chunks of 64 tokens (three passes: each chunk's own
@@ -1624,7 +1630,7 @@ def gated_recurrence(x: torch.Tensor, columns: dict, heads: int, dim: int, value
     for name, w in (("q", heads * dim), ("k", heads * dim), ("v", heads * value_dim)) + (
             (("i", heads), ("f", heads)) if mode == "exp_gates" else ()):
         c = columns[name]
-        if c < 0 or c + w > ld:
+        if c < 0 or (c % ld) + w > ld or c // ld > rows_below:
             raise ValueError(f"columns of {name!r} ({c} .. {c + w}) lie outside the matrix of width {ld}")
     for v_, nm in ((batch.row_start, "row_start"), (batch.starts, "starts"), (batch.state_slots, "state_slots")):
         _dev(v_, nm, I32, 1)
@@ -1637,6 +1643,10 @@ def gated_recurrence(x: torch.Tensor, columns: dict, heads: int, dim: int, value
     bias = i_bias if i_bias is not None else f_bias
     lib = library()
     lens = getattr(batch, "row_lens", None)
+    if rows_below:
+        if rows_below < 0 or not x.is_contiguous() or x.untyped_storage().nbytes() - x.storage_offset() * 4 < (t + rows_below) * ld * 4:
+            raise ValueError(f"x is not the top of a matrix with {rows_below} more rows")
+        chunks = False  # the chunked kernels read columns of the row alone
     if mode == "wkv":
         if chunks and lens is not None and max(lens) >= WKV_CHUNKED_FROM and dim <= lib.ms_wkv_chunk_max_dim():
             per = lib.ms_wkv_chunk_tokens()

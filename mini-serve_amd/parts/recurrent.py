@@ -196,6 +196,7 @@ class WKV(_RecurrentMixer):
     NAMES = {"r": "r", "k": "k", "v": "v", "g": "g", "w1": "w1", "w2": "w2", "w0": "w0", "u": "u", "o": "o", "norm": "norm",
              "mu_r": "mu.r", "mu_k": "mu.k", "mu_v": "mu.v", "mu_g": "mu.g", "mu_w": "mu.w"}
     BLENDS = ("r", "k", "v", "g", "w")  # the order of the blends; the decay's first step is the fifth product
+    STACKED_ROWS = 16  # tokens of a step up to which r, k, v and the gate are one product of stacked blends
 
     def __init__(self, spec: PartSpec, rt):
         super().__init__(spec, rt)
@@ -204,7 +205,7 @@ class WKV(_RecurrentMixer):
         # the width of the decay's first step: a configuration may state it; else the checkpoint's tensors say it
         self.rank = int(spec["decay_rank"]) if spec.get("decay_rank") else None
         self.ld = 0
-        self.mu = self.weights = self.w2 = self.w0 = self.u = None
+        self.mu = self.weights = self.stacked = self.w2 = self.w0 = self.u = None
 
     @classmethod
     def tensors(cls, spec: PartSpec) -> dict[str, TensorSpec]:
@@ -222,9 +223,15 @@ class WKV(_RecurrentMixer):
 
     def bind(self, tensors) -> None:
         n = self.names
-        self.weights = [tensors[n[k]] for k in ("r", "k", "v", "g", "w1")]
-        if len({t.dtype for t in self.weights}) != 1:
+        parts = [tensors[n[k]] for k in ("r", "k", "v", "g", "w1")]
+        if len({t.dtype for t in parts}) != 1:
             raise ValueError(f"{n['r']} and its neighbours are stored in different dtypes")
+        # r, k, v and the gate stacked: a step of few tokens multiplies its stacked blends by all of them at once (each
+        # blend by every weight: four times the multiply-adds, the weights read once, two launches for eight) and reads
+        # each projection off its own block of rows; the single weights are the stacked one's runs of rows, no copies
+        self.stacked = torch.cat(parts[:4], dim=0).contiguous()
+        rows = parts[0].shape[0]
+        self.weights = [self.stacked[i * rows : (i + 1) * rows] for i in range(4)] + [parts[4]]
         dtype = self.weights[0].dtype
         self.rank = self.weights[4].shape[0]
         if tensors[n["w2"]].shape[1] != self.rank:
@@ -247,14 +254,24 @@ class WKV(_RecurrentMixer):
 
     def forward(self, x, batch, cache, state, residual):
         ops = self.rt.ops
-        c, n = self.columns, self.heads * self.dim
+        c, n, t = self.columns, self.heads * self.dim, x.shape[0]
         blends = ops.token_shift_mix(ops.cast(x, self.mu.dtype), self.mu, state["shift"], batch)
-        x32 = torch.empty((x.shape[0], self.ld), dtype=torch.float32, device=x.device)
-        for i, (k, w) in enumerate(zip(("q", "k", "v", "g"), self.weights)):
-            ops.linear(blends[i], w, out=x32[:, c[k] : c[k] + w.shape[0]])
         decay = ops.channel_decay(ops.linear(blends[4], self.weights[4], out_dtype=torch.float32), self.w2, self.w0, log=True)
-        o = ops.gated_recurrence(x32, c, self.heads, self.dim, self.dim, batch, state, mode="wkv", channel_decay=decay, bonus=self.u)
-        y = ops.group_rmsnorm_gate(o, self.dim, self.norm, x32[:, c["g"] : c["g"] + n], self.eps, self.rt.dtype, "silu")
+        if t <= self.STACKED_ROWS and self.stacked.dtype == torch.bfloat16:
+            # block j of rows holds every product of blend j; the one that is wanted of it is its j-th run of columns
+            all32 = ops.linear(blends[:4].reshape(4 * t, self.hidden), self.stacked, out_dtype=torch.float32)
+            ld = 4 * n
+            at = {k: j * t * ld + j * n for j, k in enumerate(("q", "k", "v"))}
+            gate = all32[3 * t :, 3 * n :]
+            o = ops.gated_recurrence(all32[:t], at, self.heads, self.dim, self.dim, batch, state, mode="wkv", channel_decay=decay,
+                                     bonus=self.u, rows_below=3 * t)
+        else:
+            x32 = torch.empty((t, self.ld), dtype=torch.float32, device=x.device)
+            for i, (k, w) in enumerate(zip(("q", "k", "v", "g"), self.weights)):
+                ops.linear(blends[i], w, out=x32[:, c[k] : c[k] + w.shape[0]])
+            gate = x32[:, c["g"] : c["g"] + n]
+            o = ops.gated_recurrence(x32, c, self.heads, self.dim, self.dim, batch, state, mode="wkv", channel_decay=decay, bonus=self.u)
+        y = ops.group_rmsnorm_gate(o, self.dim, self.norm, gate, self.eps, self.rt.dtype, "silu")
         return ops.linear(y, self.o, accumulate_into=residual, defer=True)
 
     def parameters_bytes(self) -> int:
