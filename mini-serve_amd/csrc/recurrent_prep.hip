@@ -117,7 +117,9 @@ template <typename TB>
 __global__ void neg_exp_bias_kernel(float* __restrict__ z, const TB* __restrict__ b, size_t n, int C, int as_decay) {
   const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
-  const float l = -expf(z[i] + to_f32(b[i % C]));
+  // (not below -200: the decay is zero in float32 from -104 on, and sums of such logarithms over a chunk of tokens keep
+  // differences that are sharp in double precision)
+  const float l = fmaxf(-expf(z[i] + to_f32(b[i % C])), -200.f);
   z[i] = as_decay ? expf(l) : l;
 }
 

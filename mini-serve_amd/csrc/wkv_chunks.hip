@@ -12,8 +12,11 @@
 // Every exponent is a sum of log decays and so at most zero: nothing is ever divided by a decay. All float32; sums are
 // reassociated against the token-by-token kernel (which multiplies by exp(l_t) token after token), nothing else differs;
 // the exponentials are the hardware's exp2 of a float32 product (an error of a unit or two in the last place).
-// The running sums are float32: where they are large the decays they stand for are next to nothing. Head sizes up to
-// WKV_CHUNK_MAX_DIM; larger ones take the token-by-token kernel.
+// The running sums are double precision: the kernels need their differences, and the difference of two sums that both hold
+// one token's log of -100 (a channel that forgets everything there) must still be sharp for the tokens behind it; a float32
+// sum of that size would leave those differences with an error of 1e-5. Logs arrive clamped at -200 a token (the decay is
+// zero in float32 from -104 on), so a chunk's sums stay below 12,800. Head sizes up to WKV_CHUNK_MAX_DIM; larger ones take
+// the token-by-token kernel.
 #include "common.h"
 
 #define WKV_CHUNK 64
@@ -54,19 +57,20 @@ __device__ __forceinline__ void wkv_find_chunk(const int* __restrict__ row_start
 }
 
 // dst[d][t] = x[first + t][col + d] for t < count, d < D; zero elsewhere ([DP][WKV_CS]).
-__device__ __forceinline__ void wkv_load_transposed(float* dst, const float* __restrict__ x, int ld, int col, int first, int count, int D,
+template <typename TD>
+__device__ __forceinline__ void wkv_load_transposed(TD* dst, const float* __restrict__ x, int ld, int col, int first, int count, int D,
                                                     int DP) {
   for (int i = threadIdx.x; i < DP * WKV_CHUNK; i += 256) {
     const int t = i / DP, d = i % DP;  // consecutive threads read consecutive columns of one token
-    dst[d * WKV_CS + t] = (t < count && d < D) ? x[(size_t)(first + t) * ld + col + d] : 0.f;
+    dst[d * WKV_CS + t] = (TD)((t < count && d < D) ? x[(size_t)(first + t) * ld + col + d] : 0.f);
   }
 }
 
 // In place over L [DP][WKV_CS] of log decays: the running sums A_t (inclusive). A thread per channel, in token order.
-__device__ __forceinline__ void wkv_running_sums(float* L, int DP) {
+__device__ __forceinline__ void wkv_running_sums(double* L, int DP) {
   if (threadIdx.x < DP) {
-    float* row = L + threadIdx.x * WKV_CS;
-    float run = 0.f;
+    double* row = L + threadIdx.x * WKV_CS;
+    double run = 0.0;
     for (int t = 0; t < WKV_CHUNK; ++t) {
       run += row[t];
       row[t] = run;
@@ -80,7 +84,7 @@ __global__ __launch_bounds__(256) void wkv_chunk_summary_kernel(WkvChunkArgs a) 
   const int DP = (D + 3) & ~3;
   float* Kw = sm;                   // [WKV_CHUNK][DP]: keys times what is left of them at the chunk's end
   float* V = Kw + WKV_CHUNK * DP;   // [WKV_CHUNK][DP]
-  float* A = V + WKV_CHUNK * DP;    // [DP][WKV_CS]
+  double* A = reinterpret_cast<double*>(V + WKV_CHUNK * DP);  // [DP][WKV_CS] (8-byte aligned: both tiles are multiples of 4 floats)
   int row, first, count, base;
   wkv_find_chunk(a.row_start, a.rows, blockIdx.x, &row, &first, &count, &base);
   wkv_load_transposed(A, a.lw, a.ld_w, h * D, first, count, D, DP);
@@ -96,10 +100,10 @@ __global__ __launch_bounds__(256) void wkv_chunk_summary_kernel(WkvChunkArgs a) 
   __syncthreads();
   for (int i = tid; i < WKV_CHUNK * DP; i += 256) {
     const int t = i / DP, d = i % DP;
-    Kw[i] *= __expf(A[d * WKV_CS + WKV_CHUNK - 1] - A[d * WKV_CS + t]);  // tokens past the count hold zero keys and zero logs
+    Kw[i] *= __expf((float)(A[d * WKV_CS + WKV_CHUNK - 1] - A[d * WKV_CS + t]));  // tokens past the count hold zero keys and zero logs
   }
   const size_t at = (size_t)blockIdx.x * a.H + h;
-  if (tid < D) a.G[at * D + tid] = __expf(A[tid * WKV_CS + WKV_CHUNK - 1]);
+  if (tid < D) a.G[at * D + tid] = __expf((float)A[tid * WKV_CS + WKV_CHUNK - 1]);
   __syncthreads();
   // U[d][e]: 4 x 4 outputs a thread
   const int tiles = DP / 4;
@@ -170,11 +174,11 @@ __global__ __launch_bounds__(256) void wkv_chunk_output_kernel(WkvChunkArgs a) {
   constexpr int C = WKV_CHUNK, CP = WKV_CHUNK + 4, CS = WKV_CS;
   const int D = a.D, h = blockIdx.y, tid = threadIdx.x;
   const int DP = (D + 3) & ~3;
-  float* R = sm;              // [DP][CS]: r transposed; later r * exp(B)
+  double* A = reinterpret_cast<double*>(sm);  // [DP][CS]: running sums, inclusive
+  double* Bx = A + DP * CS;                   // [DP][CS]: running sums, exclusive
+  float* R = reinterpret_cast<float*>(Bx + DP * CS);  // [DP][CS]: r transposed; later r * exp(B)
   float* K = R + DP * CS;     // [DP][CS]
-  float* A = K + DP * CS;     // [DP][CS]: running sums, inclusive
-  float* Bx = A + DP * CS;    // [DP][CS]: running sums, exclusive
-  float* V = Bx + DP * CS;    // [C][DP]
+  float* V = K + DP * CS;     // [C][DP]
   float* P = V + C * DP;      // [C][CP]
   float* us = P + C * CP;     // [DP]
   int row, first, count, base;
@@ -189,9 +193,9 @@ __global__ __launch_bounds__(256) void wkv_chunk_output_kernel(WkvChunkArgs a) {
   if (tid < DP) us[tid] = tid < D ? a.u[h * D + tid] : 0.f;
   __syncthreads();
   if (tid < DP) {
-    float run = 0.f;
+    double run = 0.0;
     for (int t = 0; t < C; ++t) {
-      const float l = Bx[tid * CS + t];
+      const double l = Bx[tid * CS + t];
       Bx[tid * CS + t] = run;
       run += l;
       A[tid * CS + t] = run;
@@ -206,11 +210,11 @@ __global__ __launch_bounds__(256) void wkv_chunk_output_kernel(WkvChunkArgs a) {
     if (j0 <= t0 + 3 && t0 < count) {
       for (int d = 0; d < D; ++d) {
         const float4 r4 = *reinterpret_cast<const float4*>(R + d * CS + t0);
-        const float4 b4 = *reinterpret_cast<const float4*>(Bx + d * CS + t0);
         const float4 k4 = *reinterpret_cast<const float4*>(K + d * CS + j0);
-        const float4 a4 = *reinterpret_cast<const float4*>(A + d * CS + j0);
-        const float rr[4] = {r4.x, r4.y, r4.z, r4.w}, bb[4] = {b4.x, b4.y, b4.z, b4.w};
-        const float kk[4] = {k4.x, k4.y, k4.z, k4.w}, aa[4] = {a4.x, a4.y, a4.z, a4.w};
+        const double2 b01 = *reinterpret_cast<const double2*>(Bx + d * CS + t0), b23 = *reinterpret_cast<const double2*>(Bx + d * CS + t0 + 2);
+        const double2 a01 = *reinterpret_cast<const double2*>(A + d * CS + j0), a23 = *reinterpret_cast<const double2*>(A + d * CS + j0 + 2);
+        const float rr[4] = {r4.x, r4.y, r4.z, r4.w}, kk[4] = {k4.x, k4.y, k4.z, k4.w};
+        const double bb[4] = {b01.x, b01.y, b23.x, b23.y}, aa[4] = {a01.x, a01.y, a23.x, a23.y};
         const float ud = us[d];
 #pragma unroll
         for (int i = 0; i < 4; ++i)
@@ -218,7 +222,7 @@ __global__ __launch_bounds__(256) void wkv_chunk_output_kernel(WkvChunkArgs a) {
           for (int j = 0; j < 4; ++j) {
             const int t = t0 + i, jj = j0 + j;
             // j < t: what is left of key j's channel when token t reads it; j == t: the bonus; j > t: nothing
-            const float wgt = jj < t ? __expf(bb[i] - aa[j]) : (jj == t ? ud : 0.f);
+            const float wgt = jj < t ? __expf((float)(bb[i] - aa[j])) : (jj == t ? ud : 0.f);
             acc[i][j] = fmaf(rr[i] * kk[j], wgt, acc[i][j]);
           }
       }
@@ -230,7 +234,7 @@ __global__ __launch_bounds__(256) void wkv_chunk_output_kernel(WkvChunkArgs a) {
   __syncthreads();
   for (int i = tid; i < DP * C; i += 256) {  // what of the state before the chunk token t still reads
     const int at = (i / C) * CS + i % C;
-    R[at] *= __expf(Bx[at]);
+    R[at] *= __expf((float)Bx[at]);
   }
   __syncthreads();
   // The state before the chunk takes the keys' place in LDS: [D][DP], zero beyond D.
@@ -294,8 +298,8 @@ extern "C" int ms_wkv_chunked(const float* x, int ld, int r_off, int k_off, int 
   if (D > WKV_CHUNK_MAX_DIM || H > 65535 || rows > 65535) return MS_UNSUPPORTED;
   WkvChunkArgs a{x, ld, r_off, k_off, v_off, H, D, lw, ld_w, u, S, row_start, starts, state_slots, out, U, G, rows};
   const int DP = (D + 3) & ~3;
-  const size_t lds1 = sizeof(float) * (size_t)(2 * WKV_CHUNK * DP + DP * WKV_CS);
-  const size_t lds3 = sizeof(float) * (size_t)(4 * DP * WKV_CS + WKV_CHUNK * DP + WKV_CHUNK * (WKV_CHUNK + 4) + DP);
+  const size_t lds1 = sizeof(float) * (size_t)(2 * WKV_CHUNK * DP + 2 * DP * WKV_CS);  // a double takes two floats' room
+  const size_t lds3 = sizeof(float) * (size_t)(6 * DP * WKV_CS + WKV_CHUNK * DP + WKV_CHUNK * (WKV_CHUNK + 4) + DP);
   if (hipFuncSetAttribute((const void*)wkv_chunk_summary_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds1) != hipSuccess ||
       hipFuncSetAttribute((const void*)wkv_chunk_output_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds3) != hipSuccess)
     return MS_LAUNCH_FAILED;

@@ -280,6 +280,10 @@ def test_decay_per_channel(channels, rank):
         close(o.channel_decay(dev(a), dev(w2), dev(w0), log=True), np.log(want), torch.float32, tol=2e-5)
         w0b = rounded(w0, torch.bfloat16)
         close(o.channel_decay(dev(a), dev(w2), dev(w0, torch.bfloat16)), np.exp(-np.exp(np.tanh(a) @ w2.T + w0b)), torch.float32, tol=2e-5)
+    # a decay of nothing: its logarithm stays a number, so that sums and differences of such logarithms do
+    huge = o.channel_decay(dev(np.zeros((2, rank))), dev(np.zeros((channels, rank))), dev(np.full(channels, 200.0)), log=True)
+    assert (huge == -200).all()
+    assert not o.channel_decay(dev(np.zeros((2, rank))), dev(np.zeros((channels, rank))), dev(np.full(channels, 200.0))).any()
 
 
 def plain_wkv(r, k, v, w, u):
@@ -308,6 +312,8 @@ def test_recurrence_with_a_decay_per_channel_and_a_bonus(heads, dim):
         r, k, v = (rng.normal(size=(T, heads, dim)) for _ in range(3))
         w = np.exp(-np.exp(rng.normal(size=(T, heads, dim)) - 1.5))
         w[:, :, 0] = 0.9995
+        w[:, :, 1] = 0.0  # a channel that keeps nothing (its logarithm arrives as -200)
+        w[5::7, :, 2] = 0.0  # ... and one that forgets everything now and then
         k[2, :, 0] = 30.0
         seqs.append((r, k, v, w))
     u = rng.normal(size=(heads, dim)) + 0.5
@@ -332,7 +338,7 @@ def test_recurrence_with_a_decay_per_channel_and_a_bonus(heads, dim):
                 x[off : off + c, 4 : 4 + 3 * n] = np.concatenate([r, k, v], axis=1)
                 wd[off : off + c] = w
                 off += c
-            out = o.gated_recurrence(dev(x), cols, heads, dim, dim, b, {"S": S}, mode="wkv", channel_decay=dev(np.log(wd)), bonus=dev(u))
+            out = o.gated_recurrence(dev(x), cols, heads, dim, dim, b, {"S": S}, mode="wkv", channel_decay=dev(np.where(wd > 0, np.log(np.maximum(wd, 1e-300)), -200.0)), bonus=dev(u))
             off = 0
             for i, c in rows:
                 got[i].append(out[off : off + c])
