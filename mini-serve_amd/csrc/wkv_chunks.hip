@@ -60,7 +60,7 @@ __device__ __forceinline__ void wkv_find_chunk(const int* __restrict__ row_start
 template <typename TD>
 __device__ __forceinline__ void wkv_load_transposed(TD* dst, const float* __restrict__ x, int ld, int col, int first, int count, int D,
                                                     int DP) {
-  for (int i = threadIdx.x; i < DP * WKV_CHUNK; i += 256) {
+  for (int i = threadIdx.x; i < DP * WKV_CHUNK; i += blockDim.x) {
     const int t = i / DP, d = i % DP;  // consecutive threads read consecutive columns of one token
     dst[d * WKV_CS + t] = (TD)((t < count && d < D) ? x[(size_t)(first + t) * ld + col + d] : 0.f);
   }
@@ -169,7 +169,9 @@ __global__ __launch_bounds__(256) void wkv_chunk_scan_kernel(WkvChunkArgs a, int
   }
 }
 
-__global__ __launch_bounds__(256) void wkv_chunk_output_kernel(WkvChunkArgs a) {
+// Five waves a block: four for the tiles below the diagonal and everything else, the fifth for the sixteen tiles on it.
+#define WKV_OUT_THREADS 320
+__global__ __launch_bounds__(WKV_OUT_THREADS) void wkv_chunk_output_kernel(WkvChunkArgs a) {
   extern __shared__ __attribute__((aligned(16))) float sm[];
   constexpr int C = WKV_CHUNK, CP = WKV_CHUNK + 4, CS = WKV_CS;
   const int D = a.D, h = blockIdx.y, tid = threadIdx.x;
@@ -186,7 +188,7 @@ __global__ __launch_bounds__(256) void wkv_chunk_output_kernel(WkvChunkArgs a) {
   wkv_load_transposed(R, a.x, a.ld, a.r_off + h * D, first, count, D, DP);
   wkv_load_transposed(K, a.x, a.ld, a.k_off + h * D, first, count, D, DP);
   wkv_load_transposed(Bx, a.lw, a.ld_w, h * D, first, count, D, DP);
-  for (int i = tid; i < C * DP; i += 256) {
+  for (int i = tid; i < C * DP; i += WKV_OUT_THREADS) {
     const int t = i / DP, d = i % DP;
     V[i] = (t < count && d < D) ? a.x[(size_t)(first + t) * a.ld + a.v_off + h * D + d] : 0.f;
   }
@@ -202,12 +204,17 @@ __global__ __launch_bounds__(256) void wkv_chunk_output_kernel(WkvChunkArgs a) {
     }
   }
   __syncthreads();
-  // P: 4 x 4 entries a thread; tiles above the diagonal hold nothing
+  // P: 4 x 4 entries a thread. A tile below the diagonal (all its keys before all its tokens) splits every exponential at
+  // the tile's last key m: exp(B_t - A_j) = exp(B_t - A_m) exp(A_m - A_j), both exponents sums of log decays and so at most
+  // zero: eight exponentials for sixteen terms. A tile on the diagonal has six terms with j < t and the bonus where j == t;
+  // those sixteen tiles are the fifth wave's, so that no wave walks both forms. Tiles above the diagonal hold nothing.
   {
-    const int ti = tid / 16, ji = tid % 16;  // 16 x 16 tiles of 4 x 4
-    const int t0 = ti * 4, j0 = ji * 4;
     float acc[4][4] = {};
-    if (j0 <= t0 + 3 && t0 < count) {
+    const bool low = tid < 256;
+    const int ti = low ? tid / 16 : tid - 256, ji = low ? tid % 16 : tid - 256;  // 16 x 16 tiles of 4 x 4
+    const int t0 = ti * 4, j0 = ji * 4;
+    const bool mine = low ? ji != ti : ti < 16;
+    if (mine && ji <= ti && t0 < count) {
       for (int d = 0; d < D; ++d) {
         const float4 r4 = *reinterpret_cast<const float4*>(R + d * CS + t0);
         const float4 k4 = *reinterpret_cast<const float4*>(K + d * CS + j0);
@@ -215,24 +222,37 @@ __global__ __launch_bounds__(256) void wkv_chunk_output_kernel(WkvChunkArgs a) {
         const double2 a01 = *reinterpret_cast<const double2*>(A + d * CS + j0), a23 = *reinterpret_cast<const double2*>(A + d * CS + j0 + 2);
         const float rr[4] = {r4.x, r4.y, r4.z, r4.w}, kk[4] = {k4.x, k4.y, k4.z, k4.w};
         const double bb[4] = {b01.x, b01.y, b23.x, b23.y}, aa[4] = {a01.x, a01.y, a23.x, a23.y};
-        const float ud = us[d];
+        if (low) {
+          float rf[4], kf[4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+          for (int i = 0; i < 4; ++i) rf[i] = rr[i] * __expf((float)(bb[i] - aa[3]));
 #pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            const int t = t0 + i, jj = j0 + j;
-            // j < t: what is left of key j's channel when token t reads it; j == t: the bonus; j > t: nothing
-            const float wgt = jj < t ? __expf((float)(bb[i] - aa[j])) : (jj == t ? ud : 0.f);
-            acc[i][j] = fmaf(rr[i] * kk[j], wgt, acc[i][j]);
-          }
+          for (int j = 0; j < 3; ++j) kf[j] = kk[j] * __expf((float)(aa[3] - aa[j]));
+          kf[3] = kk[3];
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(rf[i], kf[j], acc[i][j]);
+        } else {
+          const float ud = us[d];
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j <= i; ++j) {
+              // j < t: what is left of key j's channel when token t reads it; j == t: the bonus
+              const float wgt = j < i ? __expf((float)(bb[i] - aa[j])) : ud;
+              acc[i][j] = fmaf(rr[i] * kk[j], wgt, acc[i][j]);
+            }
+        }
       }
     }
+    if (mine)
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-      *reinterpret_cast<float4*>(P + (t0 + i) * CP + j0) = make_float4(acc[i][0], acc[i][1], acc[i][2], acc[i][3]);
+      for (int i = 0; i < 4; ++i)
+        *reinterpret_cast<float4*>(P + (t0 + i) * CP + j0) = make_float4(acc[i][0], acc[i][1], acc[i][2], acc[i][3]);
   }
   __syncthreads();
-  for (int i = tid; i < DP * C; i += 256) {  // what of the state before the chunk token t still reads
+  for (int i = tid; i < DP * C; i += WKV_OUT_THREADS) {  // what of the state before the chunk token t still reads
     const int at = (i / C) * CS + i % C;
     R[at] *= __expf((float)Bx[at]);
   }
@@ -240,7 +260,7 @@ __global__ __launch_bounds__(256) void wkv_chunk_output_kernel(WkvChunkArgs a) {
   // The state before the chunk takes the keys' place in LDS: [D][DP], zero beyond D.
   {
     const float* S0g = a.U + ((size_t)blockIdx.x * a.H + h) * (size_t)D * D;
-    for (int i = tid; i < D * DP; i += 256) {
+    for (int i = tid; i < D * DP; i += WKV_OUT_THREADS) {
       const int d = i / DP, e = i % DP;
       K[i] = e < D ? S0g[(size_t)d * D + e] : 0.f;
     }
@@ -249,7 +269,7 @@ __global__ __launch_bounds__(256) void wkv_chunk_output_kernel(WkvChunkArgs a) {
   // o[t][e]: 4 x 4 outputs a thread
   const float* S0 = K;
   const int etiles = DP / 4;
-  for (int tile = tid; tile < (C / 4) * etiles; tile += 256) {
+  for (int tile = tid; tile < (C / 4) * etiles; tile += WKV_OUT_THREADS) {
     const int t0 = (tile / etiles) * 4, e0 = (tile % etiles) * 4;
     if (t0 >= count) continue;
     float o[4][4] = {};
@@ -306,6 +326,6 @@ extern "C" int ms_wkv_chunked(const float* x, int ld, int r_off, int k_off, int 
   wkv_chunk_summary_kernel<<<dim3(chunks, H), 256, lds1, st>>>(a);
   const int slices = (D * D + 256 * 8 - 1) / (256 * 8);
   wkv_chunk_scan_kernel<<<dim3(rows, H, slices), 256, 0, st>>>(a, slices);
-  wkv_chunk_output_kernel<<<dim3(chunks, H), 256, lds3, st>>>(a);
+  wkv_chunk_output_kernel<<<dim3(chunks, H), WKV_OUT_THREADS, lds3, st>>>(a);
   return launch_status();
 }
